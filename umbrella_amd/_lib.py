@@ -1,4 +1,6 @@
-"""ctypes binding of libumbrella_hip.so (the C ABI in include/umbrella_hip.h).
+"""ctypes bindings of libumbrella_hip.so (the C ABI in include/umbrella_hip.h) and of libumbrella_seq.so (the
+sequence-mixer model family, include/umbrella_seq.h).  The two libraries are built and loaded independently: a process
+that serves only one family compiles and maps only that family's kernels.
 
 The product path has NO CPU fallback: if the HIP library is missing, or a call
 returns non-zero, this raises.  Build with ``python -c "import __graft_entry__ as g; g.build()"``.
@@ -13,7 +15,15 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("UMB_LIB_PATH") or os.path.join(_HERE, "csrc", "libumbrella_hip.so")   # override: experiments only
 
-F16, BF16 = 0, 1
+F16, BF16, F32 = 0, 1, 2
+SEQ_LIB_PATH = os.environ.get("UMB_SEQ_LIB_PATH") or os.path.join(_HERE, "csrc", "libumbrella_seq.so")
+
+
+def seq_dtype_code(dt: torch.dtype) -> int:
+    """storage dtype code of libumbrella_seq.so (it also runs in true fp32)"""
+    if dt == torch.float32:
+        return F32
+    return dtype_code(dt)
 
 
 def dtype_code(dt: torch.dtype) -> int:
@@ -188,6 +198,104 @@ SIGNATURES = {
 _VOID = {"umb_gemm_plan", "umb_gemm_plan2", "umb_ll_plan"}
 _STR = {"umb_version"}
 _SIZE = {"umb_chain_xchg_bytes"}
+
+
+
+# ---------------------------------------------------------------- libumbrella_seq.so (include/umbrella_seq.h)
+class UmbSeqLinear(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("bias", C.c_void_p), ("N", C.c_int32), ("K", C.c_int32)]
+
+
+class UmbPagedKV(C.Structure):
+    _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("kp", C.c_void_p), ("vp", C.c_void_p), ("pages", C.c_void_p),
+                ("max_pages", C.c_int32), ("page", C.c_int32), ("n_pages", C.c_int32), ("pad_", C.c_int32)]
+
+
+class UmbSeqLayer(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("has_mlp", C.c_int32), ("heads", C.c_int32), ("kv_heads", C.c_int32),
+                ("dim", C.c_int32), ("vdim", C.c_int32), ("window", C.c_int32), ("pool", C.c_int32),
+                ("rot_dims", C.c_int32), ("rank", C.c_int32), ("ff", C.c_int32), ("pad_", C.c_int32),
+                ("scale", C.c_float), ("tau", C.c_float), ("qscale", C.c_float), ("pad2_", C.c_float),
+                ("proj", UmbSeqLinear), ("a2", UmbSeqLinear), ("out", UmbSeqLinear), ("gu", UmbSeqLinear),
+                ("down", UmbSeqLinear), ("pos_bias", C.c_void_p), ("head_norm", C.c_void_p), ("norm1", C.c_void_p),
+                ("norm1b", C.c_void_p), ("norm2", C.c_void_p), ("norm2b", C.c_void_p), ("rot_freq", C.c_void_p),
+                ("kv", UmbPagedKV), ("state", C.c_void_p)]
+
+
+class UmbSeqModel(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("L", C.c_int32), ("W", C.c_int32), ("V", C.c_int32), ("groups", C.c_int32),
+                ("pad_", C.c_int32), ("eps", C.c_float), ("pad2_", C.c_float), ("embed", C.c_void_p),
+                ("final_norm", C.c_void_p), ("head", UmbSeqLinear), ("layers", C.POINTER(UmbSeqLayer))]
+
+
+class UmbSeqWork(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("h", C.c_void_p), ("proj", C.c_void_p), ("aux", C.c_void_p), ("o", C.c_void_p),
+                ("mix", C.c_void_p), ("act", C.c_void_p), ("y", C.c_void_p), ("logits", C.c_void_p),
+                ("Tmax", C.c_int32), ("Rmax", C.c_int32)]
+
+
+class UmbSeqStep(C.Structure):
+    _fields_ = [("T", C.c_int32), ("B", C.c_int32), ("R", C.c_int32), ("max_len", C.c_int32),
+                ("tokens", C.c_void_p), ("pos", C.c_void_p), ("slot", C.c_void_p), ("seq_slot", C.c_void_p),
+                ("seq_row0", C.c_void_p), ("seq_pos0", C.c_void_p), ("seq_len", C.c_void_p), ("logit_rows", C.c_void_p),
+                ("trace", C.c_void_p)]
+
+
+_PKV = C.POINTER(UmbPagedKV)
+SEQ_SIGNATURES = {
+    "umb_seq_linear": [_P, _P, _P, _P, _I, _I, _I, _I, _I],
+    "umb_seq_group_norm": [_P, _P, _P, _P, _P, _I, _I, _I, _F, _I],
+    "umb_seq_embed_norm": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I],
+    "umb_seq_resid_norm": [_P, _P, _P, _P, _P, _I, _I, _I, _F, _I],
+    "umb_gla_decay": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _F, _I],
+    "umb_gla_scan": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F],
+    "umb_gla_gate": [_P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I],
+    "umb_pwa_prep": [_P, _PKV, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I],
+    "umb_pwa_pool": [_PKV, _P, _P, _P, _I, _I, _I, _I, _I, _I],
+    "umb_pwa_attend": [_P, _P, _PKV, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I],
+    "umb_seq_forward": [C.POINTER(UmbSeqModel), C.POINTER(UmbSeqWork), C.POINTER(UmbSeqStep)],
+    "umb_argmax_rows": [_P, _P, _I, _I],
+    "umb_sample_rows": [_P, _P, _I, _I, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P],
+    "umb_seq_version": [],
+}
+_seq_lib = None
+
+
+def load_seq() -> C.CDLL:
+    """dlopen the in-tree sequence-mixer library (never a fallback)."""
+    global _seq_lib
+    if _seq_lib is not None:
+        return _seq_lib
+    if not os.path.exists(SEQ_LIB_PATH):
+        raise RuntimeError(
+            f"{SEQ_LIB_PATH} not found: the HIP extension is not built. Run __graft_entry__.build_seq() "
+            "(hipcc --offload-arch=gfx950). umbrella_amd has no CPU fallback.")
+    lib = C.CDLL(SEQ_LIB_PATH)
+    for name, args in SEQ_SIGNATURES.items():
+        fn = getattr(lib, name)
+        if name == "umb_seq_version":
+            fn.argtypes, fn.restype = [], C.c_char_p
+        else:
+            fn.argtypes, fn.restype = list(args) + [_P], C.c_int
+    _seq_lib = lib
+    return lib
+
+
+def seq_call(name: str, *args):
+    """call an entry point of libumbrella_seq.so on the current stream (tensors -> pointers, structs by reference)"""
+    lib = load_seq()
+    conv = []
+    for a in args:
+        if isinstance(a, torch.Tensor) or a is None:
+            conv.append(ptr(a))
+        elif isinstance(a, C.Structure):
+            conv.append(C.byref(a))
+        else:
+            conv.append(a)
+    rc = getattr(lib, name)(*conv, stream_ptr())
+    if rc != 0:
+        raise UmbError(f"libumbrella_seq {name} failed with code {rc}")
+
 
 _lib = None
 

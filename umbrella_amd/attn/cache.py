@@ -135,3 +135,113 @@ class TreeKVCache:
 
     def set_kv_len(self, kv_len: int):
         self.kv_offset = kv_len
+
+
+class PagedSeqCache:
+    """Paged key/value store, pooled blocks and recurrent-state slots for MANY sequences (the sequence-mixer models of
+    libumbrella_seq.so; device-side statement: csrc/seq_common.h ``pkv_tok`` / ``pkv_blk``).
+
+    * a sequence holds a SLOT (a row of the page table and of every recurrent-state array) from ``open`` to ``close``;
+    * its tokens live in PAGES of ``page`` positions handed out on demand by ``extend`` and returned by ``close``; the same
+      page numbers index every windowed-attention layer's K / V ``[pages, G, page, D]`` (storage dtype) and its pooled K / V
+      ``[pages, G, ceil(page / pool), D]`` (fp32; a block lives in the page of its last position);
+    * gated-linear-attention layers keep one fp32 state ``[slots, H, D, Dv]`` each; nothing is cleared when a slot or a page
+      is handed out again: a sequence that starts at position 0 ignores what its slot holds, and no kernel reads a cache
+      position its own sequence has not written.
+
+    Free pages and slots are LIFO stacks, so whatever was given back last is used first.
+    """
+
+    def __init__(self, kv_layers, state_layers, max_tokens: int, max_seqs: int, device, dtype, page: int = 64):
+        assert page >= 1 and max_tokens >= 1 and max_seqs >= 1
+        self.page, self.max_seqs, self.device, self.dtype = int(page), int(max_seqs), device, dtype
+        # every sequence may leave one page partly filled
+        self.n_pages = (max_tokens + page - 1) // page + max_seqs
+        self.max_pages = self.n_pages
+        self.pages_dev = torch.zeros(max_seqs, self.max_pages, dtype=torch.int32, device=device)
+        self.kv, self.state = [], []
+        for (G, D, pool) in kv_layers:
+            npb = (page + pool - 1) // pool
+            self.kv.append(dict(
+                k=torch.zeros(self.n_pages, G, page, D, dtype=dtype, device=device),
+                v=torch.zeros(self.n_pages, G, page, D, dtype=dtype, device=device),
+                kp=torch.zeros(self.n_pages, G, npb, D, dtype=torch.float32, device=device),
+                vp=torch.zeros(self.n_pages, G, npb, D, dtype=torch.float32, device=device), G=G, D=D, pool=pool))
+        for (H, D, Dv) in state_layers:
+            self.state.append(torch.zeros(max_seqs, H, D, Dv, dtype=torch.float32, device=device))
+        self.clear()
+
+    def clear(self):
+        self.free_pages = list(range(self.n_pages - 1, -1, -1))
+        self.free_slots = list(range(self.max_seqs - 1, -1, -1))
+        self.seqs = {}                                   # id -> {"slot", "len", "pages"}
+
+    # ---- bookkeeping (host)
+    def open(self, seq_id) -> int:
+        if seq_id in self.seqs:
+            raise KeyError(f"sequence {seq_id!r} is already open")
+        if not self.free_slots:
+            raise RuntimeError(f"no free sequence slot ({self.max_seqs} in use)")
+        slot = self.free_slots.pop()
+        self.seqs[seq_id] = dict(slot=slot, len=0, pages=[])
+        return slot
+
+    def close(self, seq_id):
+        s = self.seqs.pop(seq_id)
+        self.free_pages.extend(reversed(s["pages"]))
+        self.free_slots.append(s["slot"])
+
+    def length(self, seq_id) -> int:
+        return self.seqs[seq_id]["len"]
+
+    def slot(self, seq_id) -> int:
+        return self.seqs[seq_id]["slot"]
+
+    def tokens_held(self) -> int:
+        return sum(s["len"] for s in self.seqs.values())
+
+    def can_extend(self, seq_id, n: int) -> bool:
+        s = self.seqs[seq_id]
+        need = (s["len"] + n + self.page - 1) // self.page - len(s["pages"])
+        return need <= len(self.free_pages)
+
+    def extend(self, seq_id, n: int) -> int:
+        """Reserve room for the next n positions of a sequence; returns its first new position.  The page-table row on
+        the device is updated (stream-ordered) before the caller's next launch."""
+        s = self.seqs[seq_id]
+        pos0 = s["len"]
+        need = (pos0 + n + self.page - 1) // self.page - len(s["pages"])
+        if need > len(self.free_pages):
+            raise RuntimeError(f"paged cache exhausted: {need} pages wanted, {len(self.free_pages)} free "
+                               f"({self.n_pages} pages of {self.page} tokens)")
+        if need > 0:
+            have = len(s["pages"])
+            new = [self.free_pages.pop() for _ in range(need)]
+            s["pages"].extend(new)
+            self.pages_dev[s["slot"], have:have + need] = torch.tensor(new, dtype=torch.int32).to(self.device, non_blocking=False)
+        s["len"] = pos0 + n
+        return pos0
+
+    # ---- semantic access (tests, tools): never on the hot path
+    def token_rows(self, layer: int, seq_id, positions):
+        """cached (K, V) of a sequence's positions -> two tensors [len(positions), G, D]"""
+        s, c = self.seqs[seq_id], self.kv[layer]
+        pos = torch.as_tensor(positions, dtype=torch.long)
+        pg = torch.tensor(s["pages"], dtype=torch.long)[pos // self.page].to(self.device)
+        off = (pos % self.page).to(self.device)
+        return c["k"][pg, :, off], c["v"][pg, :, off]
+
+    def pooled_rows(self, layer: int, seq_id, blocks):
+        """pooled (K, V) of a sequence's blocks -> two fp32 tensors [len(blocks), G, D]"""
+        s, c = self.seqs[seq_id], self.kv[layer]
+        e = torch.as_tensor(blocks, dtype=torch.long) * c["pool"] + c["pool"] - 1
+        pg = torch.tensor(s["pages"], dtype=torch.long)[e // self.page].to(self.device)
+        idx = ((e % self.page) // c["pool"]).to(self.device)
+        return c["kp"][pg, :, idx], c["vp"][pg, :, idx]
+
+    def struct(self, layer: int) -> "_lib.UmbPagedKV":
+        c = self.kv[layer]
+        kv = _lib.UmbPagedKV()
+        kv.k, kv.v, kv.kp, kv.vp = c["k"].data_ptr(), c["v"].data_ptr(), c["kp"].data_ptr(), c["vp"].data_ptr()
+        kv.pages, kv.max_pages, kv.page, kv.n_pages = self.pages_dev.data_ptr(), self.max_pages, self.page, self.n_pages
+        return kv

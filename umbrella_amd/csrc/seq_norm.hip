@@ -1,0 +1,115 @@
+// Grouped RMS norm and the residual seams of the sequence-mixer stacks.  The residual stream is fp32; every sum of squares,
+// factor and product is fp32; only the normed activations that feed a matrix product are rounded to the storage dtype.
+//
+//   group norm: a row of W values is cut into `groups` equal consecutive parts; each part is divided by its own
+//   sqrt(mean(part^2) + eps); the whole row is multiplied by the weight.  groups == 1 is the plain RMS norm.
+//
+// One wave owns one (row, group): the three passes of the fused seam (sum y^2 | x += y f w_post, sum x^2 | h = x f' w_next)
+// touch the same elements from the same lanes, so no barrier is needed and a row's result never depends on its neighbours.
+#include "seq_common.h"
+
+template <typename P>
+__global__ __launch_bounds__(256) void group_norm_kernel(float* __restrict__ out_f32, typename El<P>::type* __restrict__ out_dt,
+                                                         const float* __restrict__ x, const int* __restrict__ rows,
+                                                         const typename El<P>::type* __restrict__ w, int W, int groups,
+                                                         float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int grp = blockIdx.y * 4 + wave;
+  if (grp >= groups) return;
+  const int t = blockIdx.x, gs = W / groups;
+  const float* xr = x + (long)(rows ? rows[t] : t) * W + (long)grp * gs;
+  float ss = 0.f;
+  for (int i = lane; i < gs; i += 64) { const float v = xr[i]; ss += v * v; }
+  ss = wave_sum(ss);
+  const float f = 1.f / sqrtf(ss / (float)gs + eps);
+  const long o = (long)t * W + (long)grp * gs;
+  for (int i = lane; i < gs; i += 64) {
+    const float v = xr[i] * f * ldf<P>(w + grp * gs + i);
+    if (out_f32) out_f32[o + i] = v;
+    if (out_dt) stf<P>(out_dt + o + i, v);
+  }
+}
+
+template <typename P>
+__global__ __launch_bounds__(256) void embed_norm_kernel(float* __restrict__ x, typename El<P>::type* __restrict__ h,
+                                                         const typename El<P>::type* __restrict__ embed,
+                                                         const int* __restrict__ tokens, const typename El<P>::type* __restrict__ w,
+                                                         int W, int V, int groups, float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int grp = blockIdx.y * 4 + wave;
+  if (grp >= groups) return;
+  const int t = blockIdx.x, gs = W / groups;
+  int tok = tokens[t];
+  tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);
+  const typename El<P>::type* er = embed + (long)tok * W + (long)grp * gs;
+  const long o = (long)t * W + (long)grp * gs;
+  float ss = 0.f;
+  for (int i = lane; i < gs; i += 64) { const float v = ldf<P>(er + i); x[o + i] = v; ss += v * v; }
+  ss = wave_sum(ss);
+  const float f = 1.f / sqrtf(ss / (float)gs + eps);
+  for (int i = lane; i < gs; i += 64) stf<P>(h + o + i, ldf<P>(er + i) * f * ldf<P>(w + grp * gs + i));
+}
+
+template <typename P>
+__global__ __launch_bounds__(256) void resid_norm_kernel(float* __restrict__ x, typename El<P>::type* __restrict__ h,
+                                                         const float* __restrict__ y, const typename El<P>::type* __restrict__ w_post,
+                                                         const typename El<P>::type* __restrict__ w_next, int W, int groups,
+                                                         float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int grp = blockIdx.y * 4 + wave;
+  if (grp >= groups) return;
+  const int t = blockIdx.x, gs = W / groups;
+  const long o = (long)t * W + (long)grp * gs;
+  float ss = 0.f;
+  for (int i = lane; i < gs; i += 64) { const float v = y[o + i]; ss += v * v; }
+  ss = wave_sum(ss);
+  const float f = 1.f / sqrtf(ss / (float)gs + eps);
+  float s2 = 0.f;
+  for (int i = lane; i < gs; i += 64) {
+    const float v = x[o + i] + y[o + i] * f * ldf<P>(w_post + grp * gs + i);
+    x[o + i] = v;
+    s2 += v * v;
+  }
+  if (!w_next) return;
+  s2 = wave_sum(s2);
+  const float f2 = 1.f / sqrtf(s2 / (float)gs + eps);
+  for (int i = lane; i < gs; i += 64) stf<P>(h + o + i, x[o + i] * f2 * ldf<P>(w_next + grp * gs + i));
+}
+
+static inline bool norm_args_ok(int T, int W, int groups) { return T >= 1 && W >= 1 && groups >= 1 && W % groups == 0; }
+
+extern "C" int umb_seq_group_norm(float* out_f32, void* out_dt, const float* x, const int* rows, const void* w, int T, int W,
+                                  int groups, float eps, int dtype, hipStream_t st) {
+  if (!norm_args_ok(T, W, groups) || !x || !w || (!out_f32 && !out_dt)) return UMB_EINVAL;
+  DISPATCH_SEQ_DTYPE(dtype, {
+    typedef typename El<P>::type E;
+    hipLaunchKernelGGL(group_norm_kernel<P>, dim3(T, (groups + 3) / 4), dim3(256), 0, st, out_f32, (E*)out_dt, x, rows,
+                       (const E*)w, W, groups, eps);
+  })
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_seq_embed_norm(float* x, void* h, const void* embed, const int* tokens, const void* w, int T, int W, int V,
+                                  int groups, float eps, int dtype, hipStream_t st) {
+  if (!norm_args_ok(T, W, groups) || !x || !h || !embed || !tokens || !w || V < 1) return UMB_EINVAL;
+  DISPATCH_SEQ_DTYPE(dtype, {
+    typedef typename El<P>::type E;
+    hipLaunchKernelGGL(embed_norm_kernel<P>, dim3(T, (groups + 3) / 4), dim3(256), 0, st, x, (E*)h, (const E*)embed, tokens,
+                       (const E*)w, W, V, groups, eps);
+  })
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_seq_resid_norm(float* x, void* h, const float* y, const void* w_post, const void* w_next, int T, int W,
+                                  int groups, float eps, int dtype, hipStream_t st) {
+  if (!norm_args_ok(T, W, groups) || !x || !y || !w_post || (w_next && !h)) return UMB_EINVAL;
+  DISPATCH_SEQ_DTYPE(dtype, {
+    typedef typename El<P>::type E;
+    hipLaunchKernelGGL(resid_norm_kernel<P>, dim3(T, (groups + 3) / 4), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
+                       (const E*)w_next, W, groups, eps);
+  })
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}

@@ -1,0 +1,228 @@
+// Sliding-window attention with mean-pooled blocks behind the window, sigmoid weights (no softmax, nothing normalised over
+// keys), over a PAGED key/value store shared by many sequences.
+//
+//   position i sees   tokens j with 0 <= i - j < window
+//              and    blocks b (positions b pool .. b pool + pool - 1) with b pool + pool - 1 <= i - window,
+//                     each through ONE key = mean of its cached keys and ONE value = mean of its cached values;
+//   tokens that left the window but whose block is not complete behind it are not seen at all.
+//   weight of a visible key = sigmoid(q.k * scale + bias[head]);  out = sigmoid(gate) * sum weight * v.
+//
+// Keys are cached AFTER rotation and unit-RMS scaling, values are the key projection as it came out of the matrix product
+// (before rotation and scaling): one projection serves both.  Rotary: interleaved pairs (2i, 2i+1) of the first rot_dims
+// features turn by angle pos * freq[i], computed in fp32 with the full-range sincosf.
+//
+// Store: pages of `page` tokens handed out by the host-side manager; per layer K, V [pages][G][page][D] in the storage
+// dtype and pooled K, V [pages][G][ceil(page / pool)][D] in fp32.  A pooled block lives in the page of its last position, so
+// it is born complete (all its tokens are cached by then, in this or earlier pages of the sequence) and dies with the
+// sequence.  The pooled mean is always taken over the cached (rounded) values in position order: the same numbers whether
+// the tokens arrived in one step or one by one.
+//
+// Because the weights are not normalised there is no running maximum and no rescaling: a query's output is a plain sum, and
+// each (token, head) sums its keys in position order per lane column -- independent of the batch and of how the prompt was cut.
+#include "seq_common.h"
+
+// ---- rotary + unit RMS + cache append.  One wave per (token, head slot); head slots 0..H-1 are queries, H..H+G-1 keys.
+template <typename P>
+__global__ __launch_bounds__(256) void pwa_prep_kernel(float* __restrict__ q, UmbPagedKV kv, const float* __restrict__ proj, int ld,
+                                                       const int* __restrict__ pos, const int* __restrict__ slot,
+                                                       const float* __restrict__ freq, int T, int H, int G, int D, int rot_dims,
+                                                       float eps) {
+  typedef typename El<P>::type E;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const long id = (long)blockIdx.x * 4 + wave;
+  if (id >= (long)T * (H + G)) return;
+  const int t = (int)(id / (H + G)), hs = (int)(id % (H + G));
+  const bool is_q = hs < H;
+  const float* src = proj + (long)t * ld + (is_q ? (long)hs * D : (long)H * D + (long)(hs - H) * D);
+  const int p = pos[t];
+  const float pf = (float)p;
+  float* qd = is_q ? q + (long)t * H * D + (long)hs * D : nullptr;
+  E* kd = nullptr;
+  E* vd = nullptr;
+  if (!is_q) {
+    const long off = pkv_tok(kv, slot[t], p, hs - H, G, D);
+    kd = reinterpret_cast<E*>(kv.k) + off;
+    vd = reinterpret_cast<E*>(kv.v) + off;
+  }
+  // pass 1: rotate pairs, sum of squares (each lane owns whole pairs: features 2m, 2m+1 for m = lane, lane + 64, ...)
+  float ss = 0.f;
+  const int pairs = (D + 1) / 2;
+  for (int m = lane; m < pairs; m += 64) {
+    const int d0 = 2 * m, d1 = 2 * m + 1;
+    float u = src[d0], v = d1 < D ? src[d1] : 0.f;
+    if (!is_q) { stf<P>(vd + d0, u); if (d1 < D) stf<P>(vd + d1, v); }
+    if (d1 < rot_dims) {
+      float sn, cs;
+      sincosf(pf * freq[m], &sn, &cs);
+      const float ru = u * cs - v * sn, rv = v * cs + u * sn;
+      u = ru; v = rv;
+    }
+    ss += u * u + (d1 < D ? v * v : 0.f);
+  }
+  ss = wave_sum(ss);
+  const float f = 1.f / sqrtf(ss / (float)D + eps);
+  for (int m = lane; m < pairs; m += 64) {
+    const int d0 = 2 * m, d1 = 2 * m + 1;
+    float u = src[d0], v = d1 < D ? src[d1] : 0.f;
+    if (d1 < rot_dims) {
+      float sn, cs;
+      sincosf(pf * freq[m], &sn, &cs);
+      const float ru = u * cs - v * sn, rv = v * cs + u * sn;
+      u = ru; v = rv;
+    }
+    if (is_q) { qd[d0] = u * f; if (d1 < D) qd[d1] = v * f; }
+    else { stf<P>(kd + d0, u * f); if (d1 < D) stf<P>(kd + d1, v * f); }
+  }
+}
+
+// ---- pooled blocks completed by this step: grid (block-in-step, sequence, kv head), one wave each
+template <typename P>
+__global__ __launch_bounds__(64) void pwa_pool_kernel(UmbPagedKV kv, const int* __restrict__ seq_slot,
+                                                      const int* __restrict__ seq_pos0, const int* __restrict__ seq_len, int G,
+                                                      int D, int pool) {
+  typedef typename El<P>::type E;
+  const int b = blockIdx.y, g = blockIdx.z, lane = threadIdx.x;
+  const int p0 = seq_pos0[b], n = seq_len[b];
+  if (n <= 0) return;
+  // blocks whose last position e = blk pool + pool - 1 lies in [p0, p0 + n): blk >= ceil((p0 - pool + 1) / pool) = p0 / pool
+  const int first = p0 / pool;
+  const int blk = first + blockIdx.x;
+  const int e = blk * pool + pool - 1;
+  if (e >= p0 + n) return;
+  const int slot = seq_slot[b];
+  const long dst = pkv_blk(kv, slot, blk, pool, g, G, D);
+  const float inv = 1.f / (float)pool;
+  for (int d = lane; d < D; d += 64) {
+    float sk = 0.f, sv = 0.f;
+    for (int j = 0; j < pool; ++j) {
+      const long off = pkv_tok(kv, slot, blk * pool + j, g, G, D) + d;
+      sk += ldf<P>(reinterpret_cast<const E*>(kv.k) + off);
+      sv += ldf<P>(reinterpret_cast<const E*>(kv.v) + off);
+    }
+    kv.kp[dst + d] = sk * inv;
+    kv.vp[dst + d] = sv * inv;
+  }
+}
+
+// ---- attention: one wave per (token, head).  Score phase: lane = key (64 keys a round), each lane walks its key's D
+// features against q held in LDS.  Value phase: lane = value column; the 64 weights are broadcast one by one.
+constexpr int PWA_MAXC = 4;      // value columns per lane: Dv = D <= 256
+
+template <typename P>
+__global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* __restrict__ out, const float* __restrict__ q,
+                                                         UmbPagedKV kv, const float* __restrict__ proj, int ld, int gate_col,
+                                                         const typename El<P>::type* __restrict__ pos_bias,
+                                                         const int* __restrict__ pos, const int* __restrict__ slot_, int T, int H,
+                                                         int G, int D, int window, int pool, float scale) {
+  typedef typename El<P>::type E;
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int Dp = (D + 1) & ~1;                        // keeps the 8-byte offsets aligned
+  float* q_s = lds + (long)wave * (Dp + 64 + 128);  // [D] query, [64] weights, [64] 64-bit element offsets
+  float* w_s = q_s + Dp;
+  long* off_s = reinterpret_cast<long*>(w_s + 64);
+  const long id = (long)blockIdx.x * 4 + wave;
+  if (id >= (long)T * H) return;
+  const int t = (int)(id / H), h = (int)(id % H);
+  const int g = h / (H / G);
+  const int i = pos[t], slot = slot_[t];
+  for (int d = lane; d < D; d += 64) q_s[d] = q[(long)t * H * D + (long)h * D + d];
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  const float bias = pos_bias ? ldf<P>(pos_bias + h) : 0.f;
+  const int j_lo = i - window + 1 > 0 ? i - window + 1 : 0;
+  const int n_tok = i - j_lo + 1;
+  const int n_blk = i - window + 1 >= pool ? (i - window + 1) / pool : 0;
+  const int n_keys = n_blk + n_tok;
+  float acc[PWA_MAXC];
+#pragma unroll
+  for (int c = 0; c < PWA_MAXC; ++c) acc[c] = 0.f;
+  // wave-wide LDS traffic below is ordered by the wave's own program order (one wave = one instruction stream)
+  for (int base = 0; base < n_keys; base += 64) {
+    const int kx = base + lane;
+    float wgt = 0.f;
+    long off = -1;
+    bool pooled = false;
+    if (kx < n_keys) {
+      pooled = kx < n_blk;
+      off = pooled ? pkv_blk(kv, slot, kx, pool, g, G, D) : pkv_tok(kv, slot, j_lo + (kx - n_blk), g, G, D);
+      float s = 0.f;
+      if (pooled) {
+        const float* kr = kv.kp + off;
+        for (int d = 0; d < D; ++d) s += q_s[d] * kr[d];
+      } else {
+        const E* kr = reinterpret_cast<const E*>(kv.k) + off;
+        for (int d = 0; d < D; ++d) s += q_s[d] * ldf<P>(kr + d);
+      }
+      wgt = 1.f / (1.f + expf(-(s * scale + bias)));
+    }
+    w_s[lane] = wgt;
+    off_s[lane] = pooled ? ~off : off;           // pooled entries are flagged by the complement (off >= 0 always)
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const int cnt = n_keys - base < 64 ? n_keys - base : 64;
+    for (int jj = 0; jj < cnt; ++jj) {
+      const float wj = w_s[jj];
+      const long oj = off_s[jj];
+#pragma unroll
+      for (int c = 0; c < PWA_MAXC; ++c) {
+        const int d = lane + 64 * c;
+        if (d < D) acc[c] += wj * (oj < 0 ? kv.vp[~oj + d] : ldf<P>(reinterpret_cast<const E*>(kv.v) + oj + d));
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  const float gate = 1.f / (1.f + expf(-proj[(long)t * ld + gate_col + h]));
+#pragma unroll
+  for (int c = 0; c < PWA_MAXC; ++c) {
+    const int d = lane + 64 * c;
+    if (d < D) stf<P>(out + (long)t * H * D + (long)h * D + d, acc[c] * gate);
+  }
+}
+
+static inline bool pkv_ok(const UmbPagedKV* kv) {
+  return kv && kv->k && kv->v && kv->kp && kv->vp && kv->pages && kv->page >= 1 && kv->max_pages >= 1;
+}
+
+extern "C" int umb_pwa_prep(float* q, const UmbPagedKV* kv, const float* proj, int ld, const int* pos, const int* slot,
+                            const float* freq, int T, int H, int G, int D, int rot_dims, float eps, int dtype, hipStream_t st) {
+  if (T < 1 || H < 1 || G < 1 || D < 1 || rot_dims < 0 || rot_dims > D || (rot_dims & 1) || !q || !pkv_ok(kv) || !proj || !pos ||
+      !slot || (rot_dims && !freq))
+    return UMB_EINVAL;
+  const long n = (long)T * (H + G);
+  DISPATCH_SEQ_DTYPE(dtype, {
+    hipLaunchKernelGGL(pwa_prep_kernel<P>, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, st, q, *kv, proj, ld, pos, slot, freq, T, H,
+                       G, D, rot_dims, eps);
+  })
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_pwa_pool(const UmbPagedKV* kv, const int* seq_slot, const int* seq_pos0, const int* seq_len, int B, int max_len,
+                            int G, int D, int pool, int dtype, hipStream_t st) {
+  if (B < 1 || max_len < 1 || G < 1 || D < 1 || pool < 1 || !pkv_ok(kv) || !seq_slot || !seq_pos0 || !seq_len) return UMB_EINVAL;
+  const int nb = max_len / pool + 1;             // at most this many blocks end inside max_len consecutive positions
+  DISPATCH_SEQ_DTYPE(dtype, {
+    hipLaunchKernelGGL(pwa_pool_kernel<P>, dim3(nb, B, G), dim3(64), 0, st, *kv, seq_slot, seq_pos0, seq_len, G, D, pool);
+  })
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_pwa_attend(void* out, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
+                              const void* pos_bias, const int* pos, const int* slot, int T, int H, int G, int D, int window,
+                              int pool, float scale, int dtype, hipStream_t st) {
+  if (T < 1 || H < 1 || G < 1 || H % G || D < 1 || D > 64 * PWA_MAXC || window < 1 || pool < 1 || !out || !q || !pkv_ok(kv) ||
+      !proj || !pos || !slot)
+    return UMB_EINVAL;
+  const long n = (long)T * H;
+  const size_t lds = 4 * (size_t)(((D + 1) & ~1) + 64 + 128) * sizeof(float);
+  DISPATCH_SEQ_DTYPE(dtype, {
+    typedef typename El<P>::type E;
+    hipLaunchKernelGGL(pwa_attend_kernel<P>, dim3((unsigned)((n + 3) / 4)), dim3(256), lds, st, (E*)out, q, *kv, proj, ld,
+                       gate_col, (const E*)pos_bias, pos, slot, T, H, G, D, window, pool, scale);
+  })
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}

@@ -11,11 +11,15 @@ from __future__ import annotations
 
 import os
 
-from .config import KNOWN
+from .config import KNOWN, read_architecture
+from .gitopel import Gitopel
 from .llama import Llama
 
 
 class AutoModelLM:
+    # a local directory is resolved by the architecture its config.json names; directories that name none of these are
+    # Hugging Face Llama / Qwen2 / Mistral checkpoints
+    _ARCHITECTURE_MAPPING = {"Gitopel": Gitopel}
     _MODEL_MAPPING = {name: Llama for name in KNOWN}
     _OFFLOAD_MODEL_MAPPING = dict(_MODEL_MAPPING)
     _CUDAGRAPH_MODEL_MAPPING = dict(_MODEL_MAPPING)
@@ -30,6 +34,8 @@ class AutoModelLM:
             table, what = cls._OFFLOAD_MODEL_MAPPING, " (offload)"
         if model_name in table:
             klass = table[model_name]
+        elif os.path.isdir(str(model_name)) and read_architecture(model_name) in cls._ARCHITECTURE_MAPPING:
+            klass = cls._ARCHITECTURE_MAPPING[read_architecture(model_name)]
         elif os.path.isdir(str(model_name)) and os.path.exists(os.path.join(model_name, "config.json")):
             klass = Llama
         else:

@@ -191,3 +191,64 @@ def rope_tables(cfg: LlamaCfg, max_length: int, dtype) -> tuple[torch.Tensor, to
     freqs = torch.outer(torch.arange(max_length, dtype=torch.float32), inv)
     emb = torch.cat((freqs, freqs), dim=-1)
     return (emb.cos() * scale).to(dtype), (emb.sin() * scale).to(dtype)
+
+
+# ---------------------------------------------------------------- sequence-mixer stacks (libumbrella_seq.so)
+@dataclass
+class PooledWindowAttnCfg:
+    """Sliding-window attention with mean-pooled blocks behind the window and sigmoid weights; values are the key
+    projection; grouped query heads; interleaved rotary on the first ``rot_dims`` features; unit-RMS q and k."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    window: int
+    pool: int
+    rot_dims: int
+    rot_base: float
+    scale: float
+    kind: str = "attention"
+
+
+@dataclass
+class GLACfg:
+    """Gated linear attention: per-head [dim, vdim] state, per-key-channel decay sigmoid(low-rank(h))^(1/tau)."""
+    heads: int
+    dim: int
+    vdim: int
+    tau: float
+    rank: int = 0                    # columns of the decay's down-projection: read from the tensor's shape at load
+    kind: str = "gla"
+
+
+@dataclass
+class SeqLayerCfg:
+    mixer: object                    # PooledWindowAttnCfg | GLACfg
+    ff: int = 0                      # width of the gated feed-forward; 0 = the layer has none
+
+
+@dataclass
+class SeqMixCfg:
+    vocab_size: int
+    width: int
+    norm_eps: float
+    norm_groups: int
+    layers: list
+    name: str = "seqmix"
+    architecture: str = ""
+    eos_token_id: list = field(default_factory=list)
+
+    @property
+    def num_hidden_layers(self):
+        return len(self.layers)
+
+
+def read_architecture(path: str) -> str:
+    """the ``architecture`` (or first ``architectures``) entry of a model directory's config.json, '' if none"""
+    try:
+        with open(os.path.join(path, "config.json")) as f:
+            c = json.load(f)
+    except (OSError, ValueError):
+        return ""
+    a = c.get("architecture") or (c.get("architectures") or [""])[0]
+    return a if isinstance(a, str) else ""

@@ -1,0 +1,230 @@
+"""Runtime of the sequence-mixer model family on the HIP path (libumbrella_seq.so, include/umbrella_seq.h).
+
+A model is a LIST of layers, each a token mixer -- windowed attention with pooled blocks, or gated linear attention --
+plus an optional gated feed-forward, wrapped in grouped RMS norms.  The list, every size and every constant come from a
+``SeqMixCfg`` (models/config.py); a design contributes a subclass that names its checkpoint tensors (models/gitopel.py).
+
+Unlike the tree-decoding ``Llama`` runtime this one serves MANY sequences: a step is a ragged batch (the rows of each
+sequence contiguous, nothing padded), key/value pages and recurrent-state slots are handed out by
+``attn.cache.PagedSeqCache``, and the residual stream is fp32.  ``dtype`` may be bfloat16 / float16 (weights, cached
+keys, matrix-product inputs in 16 bits; norms, scores, decays, state and accumulators in fp32) or float32 (everything).
+
+Everything numeric runs in the library; this class owns buffers and descriptors.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+from .. import _lib
+from .._lib import UmbSeqLayer, UmbSeqLinear, UmbSeqModel, UmbSeqStep, UmbSeqWork
+from ..attn.cache import PagedSeqCache
+from .base import LLMBase
+from .config import SeqMixCfg
+
+KIND_CODE = {"attention": 0, "gla": 1}
+
+
+def _linear(w, b=None) -> UmbSeqLinear:
+    s = UmbSeqLinear()
+    s.w, s.bias = w.data_ptr(), (b.data_ptr() if b is not None else None)
+    s.N, s.K = w.shape
+    return s
+
+
+class SeqMixLM(LLMBase):
+    """Subclasses provide ``read_config(path)``, ``layer_tensors(i, layer_cfg, get)`` and ``top_tensors(get)``."""
+
+    def __init__(self, model_name: str, batch_size: int = 1, max_length: int = 256, device: str = "cuda:0",
+                 dtype=torch.bfloat16, offload: bool = False, cuda_graph: bool = False, state_dict=None,
+                 config: SeqMixCfg | None = None, seed: int = 0, max_tokens: int | None = None, page_size: int = 64,
+                 max_step_tokens: int | None = None) -> None:
+        super().__init__()
+        if offload:
+            raise ValueError("sequence-mixer models are device resident (offload is not supported)")
+        self.model_name, self.device, self.dtype = model_name, device, dtype
+        self.batch_size = max(1, int(batch_size))              # sequence slots
+        self.max_length = int(max_length)                      # longest sequence
+        self.max_tokens = int(max_tokens) if max_tokens else self.batch_size * self.max_length   # tokens held by all
+        self.page_size = int(page_size)
+        self.max_step_tokens = int(max_step_tokens) if max_step_tokens else None
+        self._state, self._seed = state_dict, seed
+        if config is not None:
+            self.config = config
+        elif os.path.isdir(str(model_name)):
+            self.config = self.read_config(model_name)
+        else:
+            raise ValueError(f"'{model_name}' is not a model directory and no config was given")
+        self.eos_tokens = list(self.config.eos_token_id)
+        self.ws_tokens = self.logit_rows = 0
+
+    # ------------------------------------------------------------------ weights
+    def _getter(self):
+        dev, dt = self.device, self.dtype
+        if self._state is not None:
+            sd = self._state
+            return lambda name: sd[name].to(device=dev, dtype=dt if sd[name].is_floating_point() else None).contiguous()
+        from safetensors import safe_open
+        files = [os.path.join(self.model_name, f) for f in sorted(os.listdir(self.model_name)) if f.endswith(".safetensors")]
+        index = {}
+        for f in files:
+            with safe_open(f, "pt") as h:
+                for k in h.keys():
+                    index[k] = f
+
+        def get(name):
+            with safe_open(index[name], "pt") as h:
+                t = h.get_tensor(name)
+            return t.to(device=dev, dtype=dt if t.is_floating_point() else None).contiguous()
+        return get
+
+    def alloc(self, **kwargs):
+        c, dev, dt = self.config, self.device, self.dtype
+        _lib.load_seq()
+        get = self._getter()
+        self._top = self.top_tensors(get)
+        assert tuple(self._top["embed"].shape) == (c.vocab_size, c.width), tuple(self._top["embed"].shape)
+        L = len(c.layers)
+        self._tensors, kv_layers, state_layers = [], [], []
+        for i, ly in enumerate(c.layers):
+            t = self.layer_tensors(i, ly, get)
+            t = {k: (v.contiguous() if isinstance(v, torch.Tensor) else v) for k, v in t.items()}
+            m = ly.mixer
+            if m.kind == "attention":
+                if m.vdim != m.dim:
+                    raise ValueError("values are the key projection: vdim must equal dim")
+                if m.heads % m.kv_heads:
+                    raise ValueError("heads must be a multiple of kv_heads")
+                t["cache_index"] = len(kv_layers)
+                kv_layers.append((m.kv_heads, m.dim, m.pool))
+                i2 = torch.arange(m.rot_dims // 2, dtype=torch.float32)
+                t["rot_freq"] = (m.rot_base ** (-2 * i2 / m.rot_dims)).to(dev) if m.rot_dims else None     # fp32 frequencies
+            else:
+                t["cache_index"] = len(state_layers)
+                state_layers.append((m.heads, m.dim, m.vdim))
+            self._tensors.append(t)
+        self.kv_cache = PagedSeqCache(kv_layers, state_layers, self.max_tokens, self.batch_size, dev, dt, page=self.page_size)
+        self._layer_structs = (UmbSeqLayer * L)()
+        for i, (ly, t) in enumerate(zip(c.layers, self._tensors)):
+            s, m = self._layer_structs[i], ly.mixer
+            s.kind, s.has_mlp, s.heads, s.dim, s.vdim, s.ff = KIND_CODE[m.kind], int(ly.ff > 0), m.heads, m.dim, m.vdim, ly.ff
+            s.proj, s.out = _linear(t["proj_w"], t["proj_b"]), _linear(t["out_w"], t["out_b"])
+            s.norm1, s.norm1b = t["norm1"].data_ptr(), t["norm1b"].data_ptr()
+            if m.kind == "attention":
+                s.kv_heads, s.window, s.pool, s.rot_dims, s.scale = m.kv_heads, m.window, m.pool, m.rot_dims, m.scale
+                s.pos_bias = t["pos_bias"].data_ptr() if t.get("pos_bias") is not None else None
+                s.rot_freq = t["rot_freq"].data_ptr() if t["rot_freq"] is not None else None
+                s.kv = self.kv_cache.struct(t["cache_index"])
+            else:
+                s.rank, s.tau, s.qscale = m.rank, m.tau, float(m.dim) ** -0.5
+                s.a2, s.head_norm = _linear(t["a2_w"], t["a2_b"]), t["head_norm"].data_ptr()
+                s.state = self.kv_cache.state[t["cache_index"]].data_ptr()
+            if ly.ff:
+                s.norm2, s.norm2b = t["norm2"].data_ptr(), t["norm2b"].data_ptr()
+                s.gu, s.down = _linear(t["gu_w"]), _linear(t["down_w"])
+        mdl = self._m = UmbSeqModel()
+        mdl.dtype, mdl.L, mdl.W, mdl.V, mdl.groups, mdl.eps = _lib.seq_dtype_code(dt), L, c.width, c.vocab_size, c.norm_groups, c.norm_eps
+        mdl.embed, mdl.final_norm, mdl.head = self._top["embed"].data_ptr(), self._top["final_norm"].data_ptr(), _linear(self._top["head"])
+        mdl.layers = C.cast(self._layer_structs, C.POINTER(UmbSeqLayer))
+        self.reserve(self.max_step_tokens or 256)
+        torch.cuda.synchronize()
+
+    # ------------------------------------------------------------------ workspace
+    def reserve(self, tokens: int, logit_rows: int | None = None):
+        """Size the activation workspace for steps of up to `tokens` rows, `logit_rows` of which may ask for logits."""
+        logit_rows = logit_rows or tokens
+        if tokens <= self.ws_tokens and logit_rows <= self.logit_rows:
+            return
+        T, R = max(tokens, self.ws_tokens), max(logit_rows, self.logit_rows)
+        c, dev, dt = self.config, self.device, self.dtype
+        projN = max(t["proj_w"].shape[0] for t in self._tensors)
+        hd = max(ly.mixer.heads * ly.mixer.dim for ly in c.layers)
+        hv = max(ly.mixer.heads * ly.mixer.vdim for ly in c.layers)
+        ff = max([ly.ff for ly in c.layers] + [1])
+        f32 = torch.float32
+        b = self._bufs = dict(
+            x=torch.zeros(T, c.width, dtype=f32, device=dev), h=torch.zeros(T, c.width, dtype=dt, device=dev),
+            proj=torch.zeros(T, projN, dtype=f32, device=dev), aux=torch.zeros(T, hd, dtype=f32, device=dev),
+            o=torch.zeros(T, hv, dtype=f32, device=dev), mix=torch.zeros(T, hv, dtype=dt, device=dev),
+            act=torch.zeros(T, ff, dtype=dt, device=dev), y=torch.zeros(T, c.width, dtype=f32, device=dev),
+            logits=torch.zeros(R, c.vocab_size, dtype=f32, device=dev))
+        ws = self._ws = UmbSeqWork()
+        for k in ("x", "h", "proj", "aux", "o", "mix", "act", "y", "logits"):
+            setattr(ws, k, b[k].data_ptr())
+        ws.Tmax, ws.Rmax = T, R
+        self.ws_tokens, self.logit_rows = T, R
+
+    @property
+    def logits_buffer(self) -> torch.Tensor:
+        return self._bufs["logits"]
+
+    # ------------------------------------------------------------------ sequences
+    def open(self, seq_id):
+        return self.kv_cache.open(seq_id)
+
+    def close(self, seq_id):
+        self.kv_cache.close(seq_id)
+
+    def clear(self):
+        self.kv_cache.clear()
+
+    # ------------------------------------------------------------------ forward
+    @torch.inference_mode()
+    def forward_batch(self, parts, want=None, trace: bool = False):
+        """One step of a ragged batch.  parts: [(seq_id, token ids)], each the NEXT tokens of an open sequence; want: per
+        part the indices (into that part) whose logits are asked for (default: the last one).  Returns the fp32 logits
+        [rows wanted, V] (a view of the workspace, valid until the next step) in the order of parts and of want; with
+        trace also the residual stream after every layer [L, T, W]."""
+        cache, dev = self.kv_cache, self.device
+        toks, pos, slot, seq_slot, row0, pos0, lens, rows = [], [], [], [], [], [], [], []
+        for i, (sid, ids) in enumerate(parts):
+            ids = [int(v) for v in (ids.tolist() if isinstance(ids, torch.Tensor) else ids)]
+            n = len(ids)
+            if n == 0:
+                raise ValueError("a part of a step needs at least one token")
+            if cache.length(sid) + n > self.max_length:
+                raise RuntimeError(f"sequence {sid!r} would exceed max_length {self.max_length}")
+            p0, sl = cache.extend(sid, n), cache.slot(sid)
+            seq_slot.append(sl), row0.append(len(toks)), pos0.append(p0), lens.append(n)
+            w = [n - 1] if want is None else list(want[i])
+            rows.extend(len(toks) + int(k) for k in w)
+            toks.extend(ids), pos.extend(range(p0, p0 + n)), slot.extend([sl] * n)
+        T, B, R = len(toks), len(parts), len(rows)
+        self.reserve(T, max(R, 1))
+        meta = torch.tensor(toks + pos + slot + seq_slot + row0 + pos0 + lens + rows, dtype=torch.int32).to(dev)
+        o = [0, T, 2 * T, 3 * T, 3 * T + B, 3 * T + 2 * B, 3 * T + 3 * B, 3 * T + 4 * B]
+        p = meta.data_ptr()
+        s = UmbSeqStep()
+        s.T, s.B, s.R, s.max_len = T, B, R, max(lens)
+        s.tokens, s.pos, s.slot, s.seq_slot, s.seq_row0, s.seq_pos0, s.seq_len, s.logit_rows = (p + 4 * v for v in o)
+        tr = torch.empty(len(self.config.layers), T, self.config.width, dtype=torch.float32, device=dev) if trace else None
+        s.trace = tr.data_ptr() if trace else None
+        self._keep = meta
+        rc = _lib.load_seq().umb_seq_forward(C.byref(self._m), C.byref(self._ws), C.byref(s), _lib.stream_ptr())
+        if rc != 0:
+            raise _lib.UmbError(f"libumbrella_seq umb_seq_forward failed with code {rc}")
+        logits = self._bufs["logits"][:R]
+        return (logits, tr) if trace else logits
+
+    # ---- the reference's single-sequence face (umbrella/models/base.py:4-32): tokens continue ONE sequence
+    _SOLO = "__solo__"
+
+    @torch.inference_mode()
+    def inference(self, input_ids, position_ids=None, attention_mask=None, storage_ids=None):
+        """input_ids [1, T] continue the model's own single sequence (positions must follow on from what it holds; the
+        mask and the storage ids of the tree runtime have no meaning here); returns fp32 logits [1, T, V]."""
+        ids = input_ids.reshape(-1).tolist()
+        if self._SOLO not in self.kv_cache.seqs:
+            self.kv_cache.open(self._SOLO)
+        if position_ids is not None:
+            assert int(position_ids.reshape(-1)[0]) == self.kv_cache.length(self._SOLO), "positions must continue the sequence"
+        return self.forward_batch([(self._SOLO, ids)], want=[list(range(len(ids)))]).clone()[None]
+
+    def graph_inference(self, input_ids, storage_ids=None, position_ids=None, attention_mask=None):
+        return self.inference(input_ids, position_ids, attention_mask, storage_ids)
+
+    def weight_bytes(self) -> int:
+        n = sum(v.numel() * v.element_size() for t in self._tensors for v in t.values() if isinstance(v, torch.Tensor))
+        return n + self._top["head"].numel() * self._top["head"].element_size()
