@@ -1,0 +1,135 @@
+"""Plain, slow torch-CPU statement of the sequence-mixer mechanisms (test infrastructure only; shares no code with
+umbrella_amd/).  One function per mechanism, written from the equations, whole sequences at a time, in float64 unless
+told otherwise.  Each takes plain tensors and numbers: no configuration objects, no cache, no batching.
+
+Notation: n tokens, H query heads, G key/value heads, D key size, E value size, X the mixer's input [n, width].
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+F = torch.float64
+
+
+def group_rms_norm(x, w, groups: int, eps: float):
+    """rows cut into `groups` equal consecutive parts, each divided by sqrt(mean(part^2) + eps); the row times w"""
+    shape = x.shape
+    parts = x.reshape(*shape[:-1], groups, shape[-1] // groups)
+    parts = parts / torch.sqrt(parts.pow(2).mean(-1, keepdim=True) + eps)
+    return parts.reshape(shape) * w
+
+
+def unit_rms(x, eps: float):
+    return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def silu(z):
+    return z * torch.sigmoid(z)
+
+
+def gated_ff(x, w_gate, w_up, w_down):
+    return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
+
+
+def rotate_interleaved(x, positions, rot_dims: int, base: float):
+    """x [n, heads, D]: features (2i, 2i+1), i < rot_dims / 2, turn by positions * base^(-2i / rot_dims); the rest pass"""
+    out = x.clone()
+    for i in range(rot_dims // 2):
+        ang = positions.to(x.dtype) * (base ** (-2.0 * i / rot_dims))
+        c, s = torch.cos(ang)[:, None], torch.sin(ang)[:, None]
+        u, v = x[..., 2 * i], x[..., 2 * i + 1]
+        out[..., 2 * i] = u * c - v * s
+        out[..., 2 * i + 1] = v * c + u * s
+    return out
+
+
+def visible_tokens(i: int, window: int):
+    """token positions position i sees"""
+    return [j for j in range(0, i + 1) if i - j < window]
+
+
+def visible_blocks(i: int, window: int, pool: int):
+    """pooled blocks position i sees: those that lie wholly before the window"""
+    return [b for b in range(0, i // pool + 1) if b * pool + pool - 1 <= i - window]
+
+
+def pooled_window_attention(X, wq, bq, wk, bk, wg, wo, bo, pos_bias, *, H, G, D, window, pool, rot_dims, base, scale, eps,
+                            cache_round=None, pos0: int = 0):
+    """Sliding-window attention with mean-pooled blocks and sigmoid weights; values are the projected keys.
+    cache_round: optional function applied to what a cache would hold (keys after rotation and unit RMS, raw values),
+    e.g. rounding to bfloat16, before they are pooled and attended.  Token t sits at position pos0 + t (pos0 > 0 only
+    makes sense for tests of the position arithmetic: nothing before pos0 exists)."""
+    n = X.shape[0]
+    pos = torch.arange(pos0, pos0 + n)
+    q = (X @ wq.T + bq).reshape(n, H, D)
+    k = (X @ wk.T + bk).reshape(n, G, D)
+    v = k.clone()
+    q = unit_rms(rotate_interleaved(q, pos, rot_dims, base), eps)
+    k = unit_rms(rotate_interleaved(k, pos, rot_dims, base), eps)
+    if cache_round is not None:
+        k, v = cache_round(k), cache_round(v)
+    gate = torch.sigmoid(X @ wg.T)                                   # [n, H]
+    out = torch.zeros(n, H, D, dtype=X.dtype)
+    for t in range(n):
+        i = pos0 + t
+        toks = [j - pos0 for j in visible_tokens(i, window) if j >= pos0]
+        blks = [b for b in visible_blocks(i, window, pool) if b * pool >= pos0]
+        for h in range(H):
+            g = h // (H // G)
+            acc = torch.zeros(D, dtype=X.dtype)
+            for b in blks:
+                lo = b * pool - pos0
+                kb, vb = k[lo:lo + pool, g].mean(0), v[lo:lo + pool, g].mean(0)
+                acc += torch.sigmoid((q[t, h] @ kb) * scale + pos_bias[h]) * vb
+            for j in toks:
+                acc += torch.sigmoid((q[t, h] @ k[j, g]) * scale + pos_bias[h]) * v[j, g]
+            out[t, h] = acc * gate[t, h]
+    return out.reshape(n, H * D) @ wo.T + bo
+
+
+def gated_linear_attention(X, wq, wk, wv, wg, wo, w_norm, wa1, wa2, ba2, *, H, D, E, tau, eps, state=None):
+    """S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with q scaled by D^-1/2 and
+    alpha = sigmoid(wa2 (wa1 x) + ba2)^(1/tau); per-head RMS norm of o times w_norm, times silu(wg x), then wo.
+    Returns (output [n, width], final state [H, D, E])."""
+    n = X.shape[0]
+    q = (X @ wq.T).reshape(n, H, D) / math.sqrt(D)
+    k = (X @ wk.T).reshape(n, H, D)
+    v = (X @ wv.T).reshape(n, H, E)
+    alpha = torch.sigmoid((X @ wa1.T) @ wa2.T + ba2).pow(1.0 / tau).reshape(n, H, D)
+    S = torch.zeros(H, D, E, dtype=X.dtype) if state is None else state.clone()
+    o = torch.zeros(n, H, E, dtype=X.dtype)
+    for t in range(n):
+        for h in range(H):
+            S[h] = alpha[t, h][:, None] * S[h] + torch.outer(k[t, h], v[t, h])
+            o[t, h] = S[h].T @ q[t, h]
+    o = unit_rms(o, eps) * w_norm
+    return (o.reshape(n, H * E) * silu(X @ wg.T)) @ wo.T, S
+
+
+def gitopel_forward(cfg: dict, sd: dict, tokens, dtype=F, cache_round=None, layers_out=None):
+    """Whole-sequence forward of a Gitopel checkpoint: cfg is the parsed config.json, sd maps tensor names to tensors.
+    Returns logits [n, vocab]."""
+    w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in sd.items()}
+    eps, groups = cfg["norm"]["eps"], cfg["norm"]["groups"]
+    x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)]
+    for i, ly in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", ly["mixer"]
+        h = group_rms_norm(x, w[p + "norm1"], groups, eps)
+        if ly["type"] == "attention":
+            y = pooled_window_attention(h, w[p + "mix.q"], w[p + "mix.q.b"], w[p + "mix.k"], w[p + "mix.k.b"], w[p + "mix.g"],
+                                        w[p + "mix.o"], w[p + "mix.o.b"], w[p + "mix.pb"], H=m["heads"], G=m["kv_heads"],
+                                        D=m["dim"], window=m["mask"]["size"], pool=m["mask"]["pool"], rot_dims=m["rot"]["dims"],
+                                        base=m["rot"]["base"], scale=m["scale"], eps=eps, cache_round=cache_round)
+        else:
+            y, _ = gated_linear_attention(h, w[p + "mix.q"], w[p + "mix.k"], w[p + "mix.v"], w[p + "mix.g"], w[p + "mix.o"],
+                                          w[p + "mix.norm"], w[p + "mix.a1"], w[p + "mix.a2"], w[p + "mix.a2.b"], H=m["heads"],
+                                          D=m["dim"], E=m["vdim"], tau=m["tau"], eps=eps)
+        x = x + group_rms_norm(y, w[p + "norm1b"], groups, eps)
+        if ly.get("mlp") is not None:
+            h = group_rms_norm(x, w[p + "norm2"], groups, eps)
+            x = x + group_rms_norm(gated_ff(h, w[p + "mlp.gate"], w[p + "mlp.up"], w[p + "mlp.down"]), w[p + "norm2b"], groups, eps)
+        if layers_out is not None:
+            layers_out.append(x.clone())
+    return group_rms_norm(x, w["final.norm"], groups, eps) @ w["head"].T
