@@ -1,0 +1,166 @@
+"""Prefill and decode throughput of the sequence-mixer family (Gitopel) at layer sizes that resemble real models, beside the
+framework's Llama runtime at equal width / feed-forward / head sizes and layer count.  Random weights, synthetic ids.
+
+    python bench.py --family gitopel [--sizes 1b,8b] [--prompt-len 2048] [--decode-steps 64] [--batch 16]
+
+or directly: python scripts/bench_seqmix.py.  One JSON line: per size, ms and tokens/s of
+  prefill   one prompt of --prompt-len tokens in one step (Llama: its chunked prompt path)
+  decode    one token per step behind that prompt, batch 1 (both) and batch --batch (Gitopel; the Llama runtime is batch 1)
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# width, ff, attention heads / kv heads / head size, GLA heads / key size / value size, window, pool, layers
+SIZES = {
+    "1b": dict(width=2048, ff=8192, heads=32, kv_heads=8, dim=64, gheads=8, gdim=128, gvdim=256, window=512, pool=16,
+               pattern="aagaag", vocab=32000),
+    "8b": dict(width=4096, ff=14336, heads=32, kv_heads=8, dim=128, gheads=16, gdim=128, gvdim=256, window=1024, pool=16,
+               pattern="aag", vocab=32000),
+}
+
+
+def gitopel_config(s):
+    layers = []
+    for ch in s["pattern"]:
+        if ch == "a":
+            layers.append({"type": "attention", "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"],
+                           "vdim": s["dim"], "mask": {"size": s["window"], "pool": s["pool"]},
+                           "rot": {"dims": s["dim"], "base": 10000.0}, "scale": s["dim"] ** -0.5},
+                           "mlp": {"ff": s["ff"], "kind": "dense"}})
+        else:
+            layers.append({"type": "gla", "mixer": {"heads": s["gheads"], "dim": s["gdim"], "vdim": s["gvdim"], "tau": 16.0},
+                           "mlp": {"ff": s["ff"], "kind": "dense"}})
+    return {"architecture": "Gitopel", "layers": layers, "norm": {"eps": 1e-6, "groups": 4}, "vocab": s["vocab"], "width": s["width"]}
+
+
+def device_state(cfg, dtype, seed=0, rank=16):
+    """random checkpoint drawn on the device in the storage dtype"""
+    from umbrella_amd.models import gitopel
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    sd = {}
+    for name, shape in gitopel.tensor_shapes(cfg, rank).items():
+        leaf = name.split(".")[-1]
+        if "norm" in leaf:
+            sd[name] = torch.ones(shape, dtype=dtype, device="cuda")
+        elif len(shape) == 1:
+            sd[name] = (0.1 * torch.randn(shape, generator=g, device="cuda")).to(dtype)
+        else:
+            sd[name] = (torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) / shape[1] ** 0.5).to(dtype)
+    return sd
+
+
+def timed(fn, reps):
+    torch.cuda.synchronize()
+    t0 = time.time()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.time() - t0) / reps * 1e3
+
+
+def bench_gitopel(s, args, dtype):
+    from umbrella_amd.models import gitopel
+    cfg = gitopel.config_from_dict(gitopel_config(s))
+    B, P, steps = args.batch, args.prompt_len, args.decode_steps
+    m = gitopel.Gitopel("bench", batch_size=B + 1, max_length=P + 2 * steps + 8, max_tokens=(B + 1) * (P + 2 * steps + 8),
+                        device="cuda:0", dtype=dtype, state_dict=device_state(cfg, dtype), config=cfg, max_step_tokens=max(P, B))
+    m.alloc()
+    ids = torch.randint(0, s["vocab"], (P,), generator=torch.Generator().manual_seed(1)).tolist()
+    out = {"weight_GB": round(m.weight_bytes() / 1e9, 3)}
+
+    def prefill():
+        m.open("p")
+        m.forward_batch([("p", ids)])
+        m.close("p")
+    prefill()
+    ms = timed(prefill, 3)
+    out["prefill"] = {"tokens": P, "ms": round(ms, 3), "tokens_per_s": round(P / ms * 1e3)}
+    for b in (1, B):
+        seqs = [f"s{i}" for i in range(b)]
+        for q in seqs:
+            m.open(q)
+        m.forward_batch([(q, ids) for q in seqs[:1]])
+        for q in seqs[1:]:                              # the other contexts one by one (bounded workspace)
+            m.forward_batch([(q, ids)])
+        step = lambda: m.forward_batch([(q, [7]) for q in seqs])  # noqa: E731
+        step()
+        ms = timed(step, steps)
+        out[f"decode_b{b}"] = {"context": P, "ms_per_step": round(ms, 4), "tokens_per_s": round(b / ms * 1e3),
+                               "weight_stream_TBs": round(m.weight_bytes() / ms / 1e9, 3)}
+        for q in seqs:
+            m.close(q)
+    return out
+
+
+def bench_llama(s, args, dtype):
+    os.environ.setdefault("UMBRELLA_SYNTHETIC", "1")
+    from umbrella_amd.models.config import LlamaCfg
+    from umbrella_amd.models.llama import Llama
+    P, steps = args.prompt_len, args.decode_steps
+    cfg = LlamaCfg(vocab_size=s["vocab"], hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=len(s["pattern"]),
+                   num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], head_dim=s["dim"], rope_scaling=None,
+                   rope_theta=10000.0, eos_token_id=[], name="llama-equal-size")
+    m = Llama("llama-equal-size", max_length=P + 2 * steps + 64, device="cuda:0", dtype=dtype, config=cfg)
+    m.alloc()
+    m.reserve(max(m.PREFILL_CHUNK, 64), logit_rows=64)
+    ids = torch.randint(0, s["vocab"], (P,), dtype=torch.int32, generator=torch.Generator().manual_seed(1)).cuda()
+    out = {"weight_GB": round(m.weight_bytes() / 1e9, 3)}
+    m.prefill_tokens(ids, 0)
+    ms = timed(lambda: m.prefill_tokens(ids, 0), 3)
+    out["prefill"] = {"tokens": P, "ms": round(ms, 3), "tokens_per_s": round(P / ms * 1e3)}
+    tok = torch.tensor([7], dtype=torch.int32, device="cuda")
+    pos = torch.tensor([P], dtype=torch.int32, device="cuda")
+    pre = torch.tensor([P], dtype=torch.int32, device="cuda")
+    step = lambda: m.forward_explicit(tok, pos, pos, pre)  # noqa: E731
+    step()
+    ms = timed(step, steps)
+    out["decode_b1"] = {"context": P, "ms_per_step": round(ms, 4), "tokens_per_s": round(1 / ms * 1e3),
+                        "weight_stream_TBs": round(m.weight_bytes() / ms / 1e9, 3)}
+    return out
+
+
+def run(args):
+    import __graft_entry__ as ge
+    ge.build()
+    dtype = torch.bfloat16
+    res = {}
+    for name in args.sizes.split(","):
+        s = SIZES[name]
+        res[name] = {"shape": {k: v for k, v in s.items()}}
+        if not args.no_gitopel:
+            res[name]["gitopel"] = bench_gitopel(s, args, dtype)
+            torch.cuda.empty_cache()
+        if not args.no_llama:
+            res[name]["llama_equal_size"] = bench_llama(s, args, dtype)
+            torch.cuda.empty_cache()
+    line = {"metric": "prefill / decode throughput, sequence-mixer family beside Llama at equal size", "unit": "tokens/s",
+            "dtype": "bf16", "data": "synthetic: random weights, random ids", "n_gpus": 1, "prompt_len": args.prompt_len,
+            "decode_steps": args.decode_steps, "batch": args.batch, "sizes": res}
+    print(json.dumps(line), flush=True)
+    return line
+
+
+def add_args(ap):
+    ap.add_argument("--sizes", default="1b,8b")
+    ap.add_argument("--decode-steps", type=int, default=64)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--no-llama", action="store_true")
+    ap.add_argument("--no-gitopel", action="store_true")
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--prompt-len", type=int, default=2048)
+    add_args(ap)
+    run(ap.parse_args())

@@ -133,7 +133,7 @@ def _run_gla(X, w, H, D, E, tau, eps, state, slot, pos0, splits):
     return torch.cat(outs)
 
 
-@pytest.mark.parametrize("H,D,E,rank,tau", [(2, 16, 8, 4, 8.0), (3, 24, 20, 5, 1.0), (1, 130, 70, 16, 32.0), (2, 7, 3, 1, 2.5)])
+@pytest.mark.parametrize("H,D,E,rank,tau", [(2, 16, 8, 4, 8.0), (3, 24, 20, 5, 1.0), (1, 130, 70, 16, 32.0), (2, 7, 3, 1, 2.5), (1, 256, 18, 3, 4.0)])
 def test_gla_alone_prefill_and_token_by_token(lib, H, D, E, rank, tau):
     from oracle import seqmix as O
     width, n, eps = 40, 37, 1e-5
@@ -168,8 +168,9 @@ def test_gla_far_token_survives_long_decoding(lib):
                                                                              "ba2")), H=H, D=D, E=E, tau=tau, eps=eps)
     state = torch.zeros(1, H, D, E, dtype=torch.float32, device="cuda:0")
     got = _run_gla(X, w, H, D, E, tau, eps, state, slot=0, pos0=0, splits=[8] + [1] * (n - 8))
-    scale = float(want.abs().max())
-    assert (got.cpu().double() - want).abs().max() < 1e-3 * scale
+    scale = float(want[50:].abs().max())                       # the quiet tail, far behind the loud token
+    assert (got.cpu().double() - want)[50:].abs().max() < 1e-3 * scale
+    assert (got.cpu().double() - want).abs().max() < 1e-4 * float(want.abs().max())
     forgot = X.clone()
     forgot[3] = 0
     lost, _ = O.gated_linear_attention(forgot.double(), *(w[k].double() for k in ("wq", "wk", "wv", "wg", "wo", "w_norm", "wa1",
@@ -230,7 +231,7 @@ def _attn_oracle(X, w, dtype, **kw):
 
 ATTN_CASES = [  # H, G, D, window, pool, rot_dims, page
     (4, 2, 16, 6, 3, 16, 4), (2, 2, 24, 5, 2, 8, 64), (3, 1, 10, 1, 1, 4, 3), (2, 1, 32, 9, 7, 32, 5), (6, 3, 8, 4, 11, 0, 4),
-    (1, 1, 70, 3, 2, 6, 7)]
+    (1, 1, 70, 3, 2, 6, 7), (8, 1, 16, 7, 2, 16, 8), (9, 3, 8, 3, 3, 8, 4)]
 
 
 @pytest.mark.parametrize("H,G,D,window,pool,rot_dims,page", ATTN_CASES)

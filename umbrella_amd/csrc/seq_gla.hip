@@ -7,8 +7,9 @@
 //
 // scan kernel: one WAVE owns four value columns of one (sequence, head): lane (r = lane % 16, c = lane / 16) keeps rows
 // r, r + 16, r + 32, ... of column c in registers, so the update is register-local and the read-out sum over rows is four
-// xor-shuffles inside 16 lanes -- no LDS, no barrier, and the order of every sum is fixed by (D) alone.  The token loop is
-// the only serial dimension; the next tokens' q / k / v / alpha are independent of the recurrence and are fetched ahead.
+// xor-shuffles inside 16 lanes, and the order of every sum is fixed by (D) alone -- a token's output never depends on how the
+// sequence was cut into steps.  The token loop is the only serial dimension; its inputs are independent of the recurrence and
+// are staged ahead through LDS in chunks of 16 tokens.
 #include "seq_common.h"
 
 template <typename P>
@@ -30,48 +31,90 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(float* __restrict__ alph
 }
 
 constexpr int GLA_MAXR = 16;     // rows per lane: D <= 256
+constexpr int GLA_TC = 16;       // tokens per staged chunk
+constexpr int GLA_COLS = 16;     // value columns per workgroup (4 per wave)
 
+// Workgroup = (sequence, head, 16 value columns), 4 waves of 4 columns.  The token loop is serial, so its inputs must not
+// cost a memory round trip per token: chunks of 16 tokens (alpha, k, q rows of the head and the 16 v columns) are staged
+// through a double-buffered LDS tile -- the global loads of chunk c + 1 are in flight while chunk c is consumed from LDS.
 template <int NR>
-__global__ __launch_bounds__(64) void gla_scan_kernel(float* __restrict__ o, float* __restrict__ state,
-                                                      const float* __restrict__ proj, int ld, const float* __restrict__ alpha,
-                                                      const int* __restrict__ seq_slot, const int* __restrict__ seq_row0,
-                                                      const int* __restrict__ seq_pos0, const int* __restrict__ seq_len, int H,
-                                                      int D, int Dv, float qscale) {
-  const int lane = threadIdx.x, r = lane & 15, c = blockIdx.x * 4 + (lane >> 4);
+__global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, float* __restrict__ state,
+                                                       const float* __restrict__ proj, int ld, const float* __restrict__ alpha,
+                                                       const int* __restrict__ seq_slot, const int* __restrict__ seq_row0,
+                                                       const int* __restrict__ seq_pos0, const int* __restrict__ seq_len, int H,
+                                                       int D, int Dv, float qscale) {
+  extern __shared__ float lds[];
+  constexpr int STG = 3 * NR + 1;                       // staged elements per thread: TC (3 D + 16) / 256 <= 3 NR + 1
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15;
+  const int cbase = blockIdx.x * GLA_COLS, cl = wave * 4 + (lane >> 4), c = cbase + cl;
   const int h = blockIdx.y, b = blockIdx.z;
   const int n = seq_len[b];
   if (n <= 0) return;
   const bool c_ok = c < Dv;
-  const int cc = c_ok ? c : 0;
   const int slot = seq_slot[b], row0 = seq_row0[b];
-  float* sp = state + (((long)slot * H + h) * D) * Dv + cc;
+  float* sp = state + (((long)slot * H + h) * D) * Dv + (c_ok ? c : 0);
   float S[NR];
   const bool fresh = seq_pos0[b] == 0;
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
     const int d = r + 16 * i;
-    S[i] = (!fresh && d < D) ? sp[(long)d * Dv] : 0.f;
+    S[i] = (!fresh && c_ok && d < D) ? sp[(long)d * Dv] : 0.f;
   }
-  const int HD = H * D;
-  const long qo = (long)h * D, ko = (long)HD + (long)h * D, vo = 2L * HD + (long)h * Dv + cc;
-  for (int t = 0; t < n; ++t) {
-    const float* pr = proj + (long)(row0 + t) * ld;
-    const float* ar = alpha + (long)(row0 + t) * HD + (long)h * D;
-    const float v = pr[vo];
-    float acc = 0.f;
+  const int HD = H * D, rowlen = 3 * D + GLA_COLS, chunk = GLA_TC * rowlen;
+  const int nch = (n + GLA_TC - 1) / GLA_TC;
+  float stage[STG];
+  auto fetch = [&](int ch) {                            // chunk ch -> registers (zeros past the sequence / the columns)
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-      const int d = r + 16 * i;
-      if (d < D) {
-        S[i] = ar[d] * S[i] + pr[ko + d] * v;
-        acc += S[i] * (pr[qo + d] * qscale);
+    for (int e = 0; e < STG; ++e) {
+      const int idx = e * 256 + tid;
+      float v = 0.f;
+      if (idx < chunk) {
+        const int tt = idx / rowlen, ci = idx - tt * rowlen, t = ch * GLA_TC + tt;
+        if (t < n) {
+          const long row = row0 + t;
+          if (ci < D) v = alpha[row * HD + (long)h * D + ci];
+          else if (ci < 2 * D) v = proj[row * ld + HD + (long)h * D + (ci - D)];
+          else if (ci < 3 * D) v = proj[row * ld + (long)h * D + (ci - 2 * D)] * qscale;
+          else if (cbase + ci - 3 * D < Dv) v = proj[row * ld + 2L * HD + (long)h * Dv + cbase + (ci - 3 * D)];
+        }
       }
+      stage[e] = v;
     }
-    acc += __shfl_xor(acc, 1, 64);
-    acc += __shfl_xor(acc, 2, 64);
-    acc += __shfl_xor(acc, 4, 64);
-    acc += __shfl_xor(acc, 8, 64);
-    if (r == 0 && c_ok) o[(long)(row0 + t) * (H * Dv) + (long)h * Dv + c] = acc;
+  };
+  auto stash = [&](float* buf) {
+#pragma unroll
+    for (int e = 0; e < STG; ++e) {
+      const int idx = e * 256 + tid;
+      if (idx < chunk) buf[idx] = stage[e];
+    }
+  };
+  fetch(0);
+  stash(lds);
+  __syncthreads();
+  for (int ch = 0; ch < nch; ++ch) {
+    const float* buf = lds + (ch & 1) * chunk;
+    if (ch + 1 < nch) fetch(ch + 1);
+    const int cnt = n - ch * GLA_TC < GLA_TC ? n - ch * GLA_TC : GLA_TC;
+    for (int tt = 0; tt < cnt; ++tt) {
+      const float* row = buf + tt * rowlen;
+      const float v = row[3 * D + cl];
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        const int d = r + 16 * i;
+        if (d < D) {
+          S[i] = row[d] * S[i] + row[D + d] * v;
+          acc += S[i] * row[2 * D + d];
+        }
+      }
+      acc += __shfl_xor(acc, 1, 64);
+      acc += __shfl_xor(acc, 2, 64);
+      acc += __shfl_xor(acc, 4, 64);
+      acc += __shfl_xor(acc, 8, 64);
+      if (r == 0 && c_ok) o[(long)(row0 + ch * GLA_TC + tt) * (H * Dv) + (long)h * Dv + c] = acc;
+    }
+    if (ch + 1 < nch) stash(lds + ((ch + 1) & 1) * chunk);
+    __syncthreads();
   }
   if (c_ok) {
 #pragma unroll
@@ -117,11 +160,15 @@ extern "C" int umb_gla_scan(float* o, float* state, const float* proj, int ld, c
                             const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int H, int D, int Dv,
                             float qscale, hipStream_t st) {
   if (B < 1 || H < 1 || D < 1 || D > 16 * GLA_MAXR || Dv < 1 || !o || !state || !proj || !alpha) return UMB_EINVAL;
-  const dim3 grid((Dv + 3) / 4, H, B);
+  const dim3 grid((Dv + GLA_COLS - 1) / GLA_COLS, H, B);
   const int nr = (D + 15) / 16;
+  const size_t lds = 2 * (size_t)GLA_TC * (3 * D + GLA_COLS) * sizeof(float);
 #define GLA_SCAN_CASE(NR)                                                                                                 \
   case NR:                                                                                                                \
-    hipLaunchKernelGGL(gla_scan_kernel<NR>, grid, dim3(64), 0, st, o, state, proj, ld, alpha, seq_slot, seq_row0, seq_pos0, \
+    if (lds > 48 * 1024 &&                                                                                                \
+        hipFuncSetAttribute((const void*)gla_scan_kernel<NR>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+      return UMB_EHIP;                                                                                                    \
+    hipLaunchKernelGGL(gla_scan_kernel<NR>, grid, dim3(256), lds, st, o, state, proj, ld, alpha, seq_slot, seq_row0, seq_pos0, \
                        seq_len, H, D, Dv, qscale);                                                                        \
     break;
   switch (nr) {

@@ -58,21 +58,30 @@ template <> __device__ __forceinline__ f32x4 mma8<F32>(const Frag8<F32>& a, cons
 
 enum { EPI_F32 = 0, EPI_DT = 1, EPI_SILU_MUL = 2 };
 
-// TT token tiles of 16 per workgroup; DUAL: a second weight matrix W2 = W + N * K (the "up" half) with its own accumulators
-template <typename P, int TT, bool VEC, bool DUAL>
+// NT output tiles x TT token tiles of 16 per workgroup (each wave holds all NT x TT accumulator tiles of its K share: one weight
+// fragment meets TT token fragments and one token fragment NT weight fragments, so a launch of many tokens moves
+// 1 / NT + 1 / TT fragment loads per MFMA instead of 1 + 1 / TT); DUAL: a second weight matrix W2 = W + N * K (the "up" half)
+// with its own accumulators (NT <= 2: the partial tiles of both halves share the 64 KiB of LDS).
+template <typename P, int NT, int TT, bool VEC, bool DUAL>
 __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_, const typename El<P>::type* __restrict__ x,
                                                          const typename El<P>::type* __restrict__ w,
                                                          const typename El<P>::type* __restrict__ bias, int T, int N, int K,
                                                          int epi) {
   typedef typename El<P>::type E;
-  __shared__ float red[DUAL ? 2 : 1][4][TT][256];
+  static_assert(!DUAL || NT <= 2, "gate and up partials of NT x TT tiles must fit the LDS");
+  __shared__ float red[DUAL ? 2 : 1][4][NT * TT][256];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int j = lane & 15, g = lane >> 4;
-  const int n_row = blockIdx.x * 16 + j;
   const int t0 = blockIdx.y * (TT * 16);
-  const bool n_ok = n_row < N;
-  const E* wrow = w + (long)(n_ok ? n_row : 0) * K;
-  const E* wrow2 = DUAL ? wrow + (long)N * K : wrow;
+  const E* wrow[NT];
+  bool n_ok[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n_row = (blockIdx.x * NT + nt) * 16 + j;
+    n_ok[nt] = n_row < N;
+    wrow[nt] = w + (long)(n_ok[nt] ? n_row : 0) * K;
+  }
+  const long half = DUAL ? (long)N * K : 0;
   const E* xrow[TT];
   bool t_ok[TT];
 #pragma unroll
@@ -81,18 +90,24 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
     t_ok[tt] = t < T;
     xrow[tt] = x + (long)(t_ok[tt] ? t : 0) * K;
   }
-  f32x4 acc[TT], acc2[TT];
+  f32x4 acc[NT][TT], acc2[NT][TT];
 #pragma unroll
-  for (int tt = 0; tt < TT; ++tt) { acc[tt] = f32x4{0.f, 0.f, 0.f, 0.f}; acc2[tt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+  for (int tt = 0; tt < TT; ++tt) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { acc[nt][tt] = f32x4{0.f, 0.f, 0.f, 0.f}; acc2[nt][tt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+  }
 
-  constexpr int UN = TT == 1 ? 4 : 2;        // 32-k steps in flight per wave
+  constexpr int UN = (NT * TT == 1) ? 4 : 2;        // 32-k steps in flight per wave
   for (int k0 = wave * 32; k0 < K; k0 += 128 * UN) {
-    Frag8<P> a[UN], a2[UN], b[UN][TT];
+    Frag8<P> a[UN][NT], a2[UN][NT], b[UN][TT];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int k = k0 + u * 128 + g * 8;
-      a[u] = load8<P, VEC>(wrow, n_ok, k, K);
-      if constexpr (DUAL) a2[u] = load8<P, VEC>(wrow2, n_ok, k, K);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        a[u][nt] = load8<P, VEC>(wrow[nt], n_ok[nt], k, K);
+        if constexpr (DUAL) a2[u][nt] = load8<P, VEC>(wrow[nt] + half, n_ok[nt], k, K);
+      }
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) b[u][tt] = load8<P, VEC>(xrow[tt], t_ok[tt], k, K);
     }
@@ -100,54 +115,64 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
     for (int u = 0; u < UN; ++u) {
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) {
-        acc[tt] = mma8<P>(a[u], b[u][tt], acc[tt]);
-        if constexpr (DUAL) acc2[tt] = mma8<P>(a2[u], b[u][tt], acc2[tt]);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          acc[nt][tt] = mma8<P>(a[u][nt], b[u][tt], acc[nt][tt]);
+          if constexpr (DUAL) acc2[nt][tt] = mma8<P>(a2[u][nt], b[u][tt], acc2[nt][tt]);
+        }
       }
     }
   }
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) {
-    *reinterpret_cast<f32x4*>(&red[0][wave][tt][lane * 4]) = acc[tt];
-    if constexpr (DUAL) *reinterpret_cast<f32x4*>(&red[1][wave][tt][lane * 4]) = acc2[tt];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      *reinterpret_cast<f32x4*>(&red[0][wave][nt * TT + tt][lane * 4]) = acc[nt][tt];
+      if constexpr (DUAL) *reinterpret_cast<f32x4*>(&red[1][wave][nt * TT + tt][lane * 4]) = acc2[nt][tt];
+    }
   }
   __syncthreads();
-  // thread (l = tid / 4, r = tid % 4) finishes output (n = 4 (l / 16) + r, token = l % 16) of every token tile
+  // thread (l = tid / 4, r = tid % 4) finishes output (n = 4 (l / 16) + r, token = l % 16) of every tile
   const int l = threadIdx.x >> 2, r = threadIdx.x & 3;
-  const int n = blockIdx.x * 16 + 4 * (l >> 4) + r;
-  if (n >= N) return;
-  const float bv = bias ? ldf<P>(bias + n) : 0.f;
-  const float bv2 = (DUAL && bias) ? ldf<P>(bias + N + n) : 0.f;
 #pragma unroll
-  for (int tt = 0; tt < TT; ++tt) {
-    const int t = t0 + tt * 16 + (l & 15);
-    if (t >= T) continue;
-    float s = red[0][0][tt][threadIdx.x];
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = (blockIdx.x * NT + nt) * 16 + 4 * (l >> 4) + r;
+    if (n >= N) continue;
+    const float bv = bias ? ldf<P>(bias + n) : 0.f;
+    const float bv2 = (DUAL && bias) ? ldf<P>(bias + N + n) : 0.f;
 #pragma unroll
-    for (int ww = 1; ww < 4; ++ww) s += red[0][ww][tt][threadIdx.x];
-    s += bv;
-    if constexpr (DUAL) {
-      float u = red[1][0][tt][threadIdx.x];
+    for (int tt = 0; tt < TT; ++tt) {
+      const int t = t0 + tt * 16 + (l & 15);
+      if (t >= T) continue;
+      float s = red[0][0][nt * TT + tt][threadIdx.x];
 #pragma unroll
-      for (int ww = 1; ww < 4; ++ww) u += red[1][ww][tt][threadIdx.x];
-      u += bv2;
-      stf<P>(reinterpret_cast<E*>(out_) + (long)t * N + n, siluf_(s) * u);
-    } else if (epi == EPI_DT) {
-      stf<P>(reinterpret_cast<E*>(out_) + (long)t * N + n, s);
-    } else {
-      reinterpret_cast<float*>(out_)[(long)t * N + n] = s;
+      for (int ww = 1; ww < 4; ++ww) s += red[0][ww][nt * TT + tt][threadIdx.x];
+      s += bv;
+      if constexpr (DUAL) {
+        float u = red[1][0][nt * TT + tt][threadIdx.x];
+#pragma unroll
+        for (int ww = 1; ww < 4; ++ww) u += red[1][ww][nt * TT + tt][threadIdx.x];
+        u += bv2;
+        stf<P>(reinterpret_cast<E*>(out_) + (long)t * N + n, siluf_(s) * u);
+      } else if (epi == EPI_DT) {
+        stf<P>(reinterpret_cast<E*>(out_) + (long)t * N + n, s);
+      } else {
+        reinterpret_cast<float*>(out_)[(long)t * N + n] = s;
+      }
     }
   }
 }
 
-template <typename P, int TT, bool VEC>
+template <typename P, int NT, int TT, bool VEC>
 static int launch_tt(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st) {
   typedef typename El<P>::type E;
-  const dim3 grid((N + 15) / 16, (T + TT * 16 - 1) / (TT * 16));
+  constexpr int NTD = NT > 2 ? 2 : NT;             // gate/up: two tile pairs at most
+  const dim3 grid((N + NT * 16 - 1) / (NT * 16), (T + TT * 16 - 1) / (TT * 16));
   if (epi == EPI_SILU_MUL)
-    hipLaunchKernelGGL((seq_linear_kernel<P, TT, VEC, true>), grid, dim3(256), 0, st, out, (const E*)x, (const E*)w, (const E*)bias,
-                       T, N, K, epi);
+    hipLaunchKernelGGL((seq_linear_kernel<P, NTD, TT, VEC, true>), dim3((N + NTD * 16 - 1) / (NTD * 16), grid.y), dim3(256), 0, st,
+                       out, (const E*)x, (const E*)w, (const E*)bias, T, N, K, epi);
   else
-    hipLaunchKernelGGL((seq_linear_kernel<P, TT, VEC, false>), grid, dim3(256), 0, st, out, (const E*)x, (const E*)w,
+    hipLaunchKernelGGL((seq_linear_kernel<P, NT, TT, VEC, false>), grid, dim3(256), 0, st, out, (const E*)x, (const E*)w,
                        (const E*)bias, T, N, K, epi);
   UMB_LAUNCH_CHECK();
   return UMB_OK;
@@ -155,9 +180,13 @@ static int launch_tt(void* out, const void* x, const void* w, const void* bias, 
 
 template <typename P, bool VEC>
 static int launch_vec(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st) {
-  if (T <= 16) return launch_tt<P, 1, VEC>(out, x, w, bias, T, N, K, epi, st);
-  if (T <= 32) return launch_tt<P, 2, VEC>(out, x, w, bias, T, N, K, epi, st);
-  return launch_tt<P, 4, VEC>(out, x, w, bias, T, N, K, epi, st);
+  if (T <= 16) return launch_tt<P, 1, 1, VEC>(out, x, w, bias, T, N, K, epi, st);
+  if (T <= 32) return launch_tt<P, 1, 2, VEC>(out, x, w, bias, T, N, K, epi, st);
+  // many tokens: the launch is bound by fragment loads per MFMA, not by weight bytes -> four output tiles per workgroup
+  // (the K order of every output is unchanged: a row's value does not depend on which variant computed it)
+  if (T > 64 && N >= 64 && sizeof(typename El<P>::type) == 2)
+    return launch_tt<P, 4, 4, VEC>(out, x, w, bias, T, N, K, epi, st);
+  return launch_tt<P, 1, 4, VEC>(out, x, w, bias, T, N, K, epi, st);
 }
 
 extern "C" int umb_seq_linear(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, int dtype,

@@ -104,11 +104,15 @@ __global__ __launch_bounds__(64) void pwa_pool_kernel(UmbPagedKV kv, const int* 
   }
 }
 
-// ---- attention: one wave per (token, head).  Score phase: lane = key (64 keys a round), each lane walks its key's D
-// features against q held in LDS.  Value phase: lane = value column; the 64 weights are broadcast one by one.
-constexpr int PWA_MAXC = 4;      // value columns per lane: Dv = D <= 256
+// ---- attention.  Workgroup = (token, RH query heads of one key/value group): the heads of a group read the same keys and
+// values, so one pass over the keys serves all of them.  The four waves take the 64-key rounds w, w + 4, ... of the key list
+// (pooled blocks first, then the window's tokens, both in position order) and their partial sums are added through LDS in
+// wave order -- which keys land in which wave depends on the query's position alone, never on the batch or on how the prompt
+// was cut.  Score phase: lane = key, 16-byte loads along the key's row against the queries held in LDS.  Value phase:
+// lane = value column, the round's weights broadcast one key at a time.
+constexpr int PWA_MAXC = 4;      // value columns per lane: D <= 256
 
-template <typename P>
+template <typename P, int RH>
 __global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* __restrict__ out, const float* __restrict__ q,
                                                          UmbPagedKV kv, const float* __restrict__ proj, int ld, int gate_col,
                                                          const typename El<P>::type* __restrict__ pos_bias,
@@ -117,67 +121,110 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* _
   typedef typename El<P>::type E;
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int Dp = (D + 1) & ~1;                        // keeps the 8-byte offsets aligned
-  float* q_s = lds + (long)wave * (Dp + 64 + 128);  // [D] query, [64] weights, [64] 64-bit element offsets
-  float* w_s = q_s + Dp;
-  long* off_s = reinterpret_cast<long*>(w_s + 64);
-  const long id = (long)blockIdx.x * 4 + wave;
-  if (id >= (long)T * H) return;
-  const int t = (int)(id / H), h = (int)(id % H);
-  const int g = h / (H / G);
+  const int Dp = (D + 3) & ~3;
+  float* q_s = lds;                                          // [RH][Dp] queries; later [4][RH][Dp] partial outputs
+  float* w_s = lds + 4 * RH * Dp + wave * (RH * 64 + 128);   // per wave: [RH][64] weights, [64] 64-bit offsets
+  long* off_s = reinterpret_cast<long*>(w_s + RH * 64);
+  const int t = blockIdx.x, h0 = blockIdx.y * RH;
+  const int g = h0 / (H / G);
   const int i = pos[t], slot = slot_[t];
-  for (int d = lane; d < D; d += 64) q_s[d] = q[(long)t * H * D + (long)h * D + d];
-  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  const float bias = pos_bias ? ldf<P>(pos_bias + h) : 0.f;
-  const int j_lo = i - window + 1 > 0 ? i - window + 1 : 0;
-  const int n_tok = i - j_lo + 1;
-  const int n_blk = i - window + 1 >= pool ? (i - window + 1) / pool : 0;
-  const int n_keys = n_blk + n_tok;
-  float acc[PWA_MAXC];
+  for (int x = threadIdx.x; x < RH * D; x += 256) q_s[(x / D) * Dp + x % D] = q[(long)t * H * D + (long)h0 * D + x];
+  float bias[RH];
 #pragma unroll
-  for (int c = 0; c < PWA_MAXC; ++c) acc[c] = 0.f;
-  // wave-wide LDS traffic below is ordered by the wave's own program order (one wave = one instruction stream)
-  for (int base = 0; base < n_keys; base += 64) {
+  for (int r = 0; r < RH; ++r) bias[r] = pos_bias ? ldf<P>(pos_bias + h0 + r) : 0.f;
+  __syncthreads();
+  const int j_lo = i - window + 1 > 0 ? i - window + 1 : 0;
+  const int n_blk = i - window + 1 >= pool ? (i - window + 1) / pool : 0;
+  const int n_keys = n_blk + (i - j_lo + 1);
+  const bool vec = (D & 7) == 0;
+  float acc[RH][PWA_MAXC];
+#pragma unroll
+  for (int r = 0; r < RH; ++r)
+#pragma unroll
+    for (int c = 0; c < PWA_MAXC; ++c) acc[r][c] = 0.f;
+  for (int base = wave * 64; base < n_keys; base += 256) {
     const int kx = base + lane;
-    float wgt = 0.f;
-    long off = -1;
+    float s[RH];
+#pragma unroll
+    for (int r = 0; r < RH; ++r) s[r] = 0.f;
+    long off = 0;
     bool pooled = false;
     if (kx < n_keys) {
       pooled = kx < n_blk;
       off = pooled ? pkv_blk(kv, slot, kx, pool, g, G, D) : pkv_tok(kv, slot, j_lo + (kx - n_blk), g, G, D);
-      float s = 0.f;
       if (pooled) {
         const float* kr = kv.kp + off;
-        for (int d = 0; d < D; ++d) s += q_s[d] * kr[d];
+        for (int d = 0; d < D; ++d) {
+          const float kd = kr[d];
+#pragma unroll
+          for (int r = 0; r < RH; ++r) s[r] += q_s[r * Dp + d] * kd;
+        }
       } else {
         const E* kr = reinterpret_cast<const E*>(kv.k) + off;
-        for (int d = 0; d < D; ++d) s += q_s[d] * ldf<P>(kr + d);
+        bool done = false;
+        if constexpr (sizeof(E) == 2) {
+          if (vec) {
+            for (int d = 0; d < D; d += 8) {
+              const u32x4 kk = *reinterpret_cast<const u32x4*>(kr + d);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float k0 = lo_f<P>(kk[e]), k1 = hi_f<P>(kk[e]);
+#pragma unroll
+                for (int r = 0; r < RH; ++r) s[r] += q_s[r * Dp + d + 2 * e] * k0 + q_s[r * Dp + d + 2 * e + 1] * k1;
+              }
+            }
+            done = true;
+          }
+        }
+        if (!done) {
+          for (int d = 0; d < D; ++d) {
+            const float kd = ldf<P>(kr + d);
+#pragma unroll
+            for (int r = 0; r < RH; ++r) s[r] += q_s[r * Dp + d] * kd;
+          }
+        }
       }
-      wgt = 1.f / (1.f + expf(-(s * scale + bias)));
     }
-    w_s[lane] = wgt;
-    off_s[lane] = pooled ? ~off : off;           // pooled entries are flagged by the complement (off >= 0 always)
+#pragma unroll
+    for (int r = 0; r < RH; ++r) w_s[r * 64 + lane] = kx < n_keys ? 1.f / (1.f + expf(-(s[r] * scale + bias[r]))) : 0.f;
+    off_s[lane] = pooled ? ~off : off;            // pooled entries are flagged by the complement (off >= 0 always)
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
     const int cnt = n_keys - base < 64 ? n_keys - base : 64;
     for (int jj = 0; jj < cnt; ++jj) {
-      const float wj = w_s[jj];
       const long oj = off_s[jj];
+      float vv[PWA_MAXC];
 #pragma unroll
       for (int c = 0; c < PWA_MAXC; ++c) {
         const int d = lane + 64 * c;
-        if (d < D) acc[c] += wj * (oj < 0 ? kv.vp[~oj + d] : ldf<P>(reinterpret_cast<const E*>(kv.v) + oj + d));
+        vv[c] = d < D ? (oj < 0 ? kv.vp[~oj + d] : ldf<P>(reinterpret_cast<const E*>(kv.v) + oj + d)) : 0.f;
+      }
+#pragma unroll
+      for (int r = 0; r < RH; ++r) {
+        const float wj = w_s[r * 64 + jj];
+#pragma unroll
+        for (int c = 0; c < PWA_MAXC; ++c) acc[r][c] += wj * vv[c];
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
-  const float gate = 1.f / (1.f + expf(-proj[(long)t * ld + gate_col + h]));
+  __syncthreads();                                  // every wave is done with the queries: their LDS becomes the partials
 #pragma unroll
-  for (int c = 0; c < PWA_MAXC; ++c) {
-    const int d = lane + 64 * c;
-    if (d < D) stf<P>(out + (long)t * H * D + (long)h * D + d, acc[c] * gate);
+  for (int r = 0; r < RH; ++r)
+#pragma unroll
+    for (int c = 0; c < PWA_MAXC; ++c) {
+      const int d = lane + 64 * c;
+      if (d < D) lds[(wave * RH + r) * Dp + d] = acc[r][c];
+    }
+  __syncthreads();
+  for (int x = threadIdx.x; x < RH * D; x += 256) {
+    const int r = x / D, d = x % D;
+    float o = lds[(0 * RH + r) * Dp + d];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) o += lds[(w * RH + r) * Dp + d];
+    const float gate = 1.f / (1.f + expf(-proj[(long)t * ld + gate_col + h0 + r]));
+    stf<P>(out + (long)t * H * D + (long)(h0 + r) * D + d, o * gate);
   }
 }
 
@@ -216,13 +263,21 @@ extern "C" int umb_pwa_attend(void* out, const float* q, const UmbPagedKV* kv, c
   if (T < 1 || H < 1 || G < 1 || H % G || D < 1 || D > 64 * PWA_MAXC || window < 1 || pool < 1 || !out || !q || !pkv_ok(kv) ||
       !proj || !pos || !slot)
     return UMB_EINVAL;
-  const long n = (long)T * H;
-  const size_t lds = 4 * (size_t)(((D + 1) & ~1) + 64 + 128) * sizeof(float);
+  const int R = H / G;
+  const int rh = R % 8 == 0 ? 8 : (R % 4 == 0 ? 4 : (R % 2 == 0 ? 2 : 1));     // heads of one group per workgroup
+  const int Dp = (D + 3) & ~3;
+  const size_t lds = ((size_t)4 * rh * Dp + 4 * (rh * 64 + 128)) * sizeof(float);
+  const dim3 grid(T, H / rh);
+#define PWA_CASE(RH)                                                                                                       \
+  case RH:                                                                                                                 \
+    hipLaunchKernelGGL((pwa_attend_kernel<P, RH>), grid, dim3(256), lds, st, (E*)out, q, *kv, proj, ld, gate_col,          \
+                       (const E*)pos_bias, pos, slot, T, H, G, D, window, pool, scale);                                    \
+    break;
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
-    hipLaunchKernelGGL(pwa_attend_kernel<P>, dim3((unsigned)((n + 3) / 4)), dim3(256), lds, st, (E*)out, q, *kv, proj, ld,
-                       gate_col, (const E*)pos_bias, pos, slot, T, H, G, D, window, pool, scale);
+    switch (rh) { PWA_CASE(8) PWA_CASE(4) PWA_CASE(2) default: PWA_CASE(1) }
   })
+#undef PWA_CASE
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }
