@@ -5,9 +5,9 @@
 // state, the products that enter it and the read-out.  The state lives in a slot array [slots][H][D][Dv] and is carried from
 // step to step; a sequence whose first row is at position 0 starts from zero whatever its slot held before.
 //
-// scan kernel: one WAVE owns four value columns of one (sequence, head): lane (r = lane % 16, c = lane / 16) keeps rows
-// r, r + 16, r + 32, ... of column c in registers, so the update is register-local and the read-out sum over rows is four
-// xor-shuffles inside 16 lanes, and the order of every sum is fixed by (D) alone -- a token's output never depends on how the
+// scan kernel: one WAVE owns four value columns of one (sequence, head): lane (r = lane % 16, c = lane / 16) keeps NR
+// consecutive rows (r NR ...) of column c in registers, so the update is register-local and the read-out sum over rows is a
+// butterfly inside 16 lanes, and the order of every sum is fixed by (D) alone -- a token's output never depends on how the
 // sequence was cut into steps.  The token loop is the only serial dimension; its inputs are independent of the recurrence and
 // are staged ahead through LDS in chunks of 16 tokens.
 #include "seq_common.h"
@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, fl
                                                        const int* __restrict__ seq_slot, const int* __restrict__ seq_row0,
                                                        const int* __restrict__ seq_pos0, const int* __restrict__ seq_len, int H,
                                                        int D, int Dv, float qscale) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr int STG = 3 * NR + 1;                       // staged elements per thread: TC (3 D + 16) / 256 <= 3 NR + 1
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15;
   const int cbase = blockIdx.x * GLA_COLS, cl = wave * 4 + (lane >> 4), c = cbase + cl;
@@ -57,28 +57,35 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, fl
   const bool fresh = seq_pos0[b] == 0;
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
-    const int d = r + 16 * i;
+    const int d = r * NR + i;
     S[i] = (!fresh && c_ok && d < D) ? sp[(long)d * Dv] : 0.f;
   }
   const int HD = H * D, rowlen = 3 * D + GLA_COLS, chunk = GLA_TC * rowlen;
   const int nch = (n + GLA_TC - 1) / GLA_TC;
   float stage[STG];
-  auto fetch = [&](int ch) {                            // chunk ch -> registers (zeros past the sequence / the columns)
+  // chunk ch -> registers.  Every load is unconditional and lands on a valid address (indices are clamped): loads that sit in
+  // divergent branches would each wait for their own round trip.  What a clamped load brings is never used: tokens past the
+  // sequence are not consumed, columns past Dv are not written, indices past the chunk are not stashed.
+  const int tt0 = tid / rowlen, ci0 = tid - tt0 * rowlen;
+  auto fetch = [&](int ch) {
+    int tt = tt0, ci = ci0;                             // (token, column) of staged element e * 256 + tid, kept incrementally
 #pragma unroll
     for (int e = 0; e < STG; ++e) {
-      const int idx = e * 256 + tid;
-      float v = 0.f;
-      if (idx < chunk) {
-        const int tt = idx / rowlen, ci = idx - tt * rowlen, t = ch * GLA_TC + tt;
-        if (t < n) {
-          const long row = row0 + t;
-          if (ci < D) v = alpha[row * HD + (long)h * D + ci];
-          else if (ci < 2 * D) v = proj[row * ld + HD + (long)h * D + (ci - D)];
-          else if (ci < 3 * D) v = proj[row * ld + (long)h * D + (ci - 2 * D)] * qscale;
-          else if (cbase + ci - 3 * D < Dv) v = proj[row * ld + 2L * HD + (long)h * Dv + cbase + (ci - 3 * D)];
-        }
+      if (e) {
+        ci += 256;
+        while (ci >= rowlen) { ci -= rowlen; ++tt; }
+        if (tt >= GLA_TC) { tt = GLA_TC - 1; ci = rowlen - 1; }      // past the chunk: any valid address
       }
-      stage[e] = v;
+      int t = ch * GLA_TC + tt;
+      t = t < n ? t : n - 1;
+      const long row = row0 + t;
+      int vc = cbase + ci - 3 * D;
+      vc = vc < Dv ? vc : Dv - 1;
+      const float* src = ci < D ? alpha + row * HD + (long)h * D + ci
+                       : ci < 2 * D ? proj + row * ld + HD + (long)h * D + (ci - D)
+                       : ci < 3 * D ? proj + row * ld + (long)h * D + (ci - 2 * D)
+                                    : proj + row * ld + 2L * HD + (long)h * Dv + vc;
+      stage[e] = *src;
     }
   };
   auto stash = [&](float* buf) {
@@ -95,31 +102,74 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, fl
     const float* buf = lds + (ch & 1) * chunk;
     if (ch + 1 < nch) fetch(ch + 1);
     const int cnt = n - ch * GLA_TC < GLA_TC ? n - ch * GLA_TC : GLA_TC;
-    for (int tt = 0; tt < cnt; ++tt) {
-      const float* row = buf + tt * rowlen;
-      const float v = row[3 * D + cl];
-      float acc = 0.f;
+    float pt[GLA_TC];                                   // this lane's share (its rows) of every token's read-out
 #pragma unroll
-      for (int i = 0; i < NR; ++i) {
-        const int d = r + 16 * i;
-        if (d < D) {
-          S[i] = row[d] * S[i] + row[D + d] * v;
-          acc += S[i] * row[2 * D + d];
+    for (int tt = 0; tt < GLA_TC; ++tt) {
+      float acc = 0.f;
+      if (tt < cnt) {
+        const float* row = buf + tt * rowlen;
+        const float v = row[3 * D + cl];
+        float al[NR], kk[NR], qq[NR];
+        bool got = false;
+        if constexpr (NR % 4 == 0) {
+          if ((D & 3) == 0) {                           // 16-byte LDS reads of the lane's NR consecutive rows
+#pragma unroll
+            for (int i = 0; i < NR; i += 4) {
+              const f32x4 a4 = *reinterpret_cast<const f32x4*>(row + r * NR + i);
+              const f32x4 k4 = *reinterpret_cast<const f32x4*>(row + D + r * NR + i);
+              const f32x4 q4 = *reinterpret_cast<const f32x4*>(row + 2 * D + r * NR + i);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) { al[i + e] = a4[e]; kk[i + e] = k4[e]; qq[i + e] = q4[e]; }
+            }
+            got = true;
+          }
+        }
+        if (!got) {
+#pragma unroll
+          for (int i = 0; i < NR; ++i) {
+            const int d = r * NR + i;
+            al[i] = row[d]; kk[i] = row[D + d]; qq[i] = row[2 * D + d];
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          if (r * NR + i < D) {
+            S[i] = al[i] * S[i] + kk[i] * v;
+            acc += S[i] * qq[i];
+          }
         }
       }
-      acc += __shfl_xor(acc, 1, 64);
-      acc += __shfl_xor(acc, 2, 64);
-      acc += __shfl_xor(acc, 4, 64);
-      acc += __shfl_xor(acc, 8, 64);
-      if (r == 0 && c_ok) o[(long)(row0 + ch * GLA_TC + tt) * (H * Dv) + (long)h * Dv + c] = acc;
+      pt[tt] = acc;
     }
+    // sum over the 16 row lanes, all 16 tokens at once: a transposing butterfly (15 exchanges instead of 64).  At the step with
+    // mask m a lane keeps the half of its values whose token bit m equals its own lane bit and hands the other half to its
+    // partner; lane r ends up with the whole sum of token r.  Every token's sum has the same tree (pairs by 8, 4, 2, 1).
+    float p8[8], p4[4], p2[2];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool up = r & 8;
+      p8[j] = (up ? pt[j + 8] : pt[j]) + __shfl_xor(up ? pt[j] : pt[j + 8], 8, 64);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool up = r & 4;
+      p4[j] = (up ? p8[j + 4] : p8[j]) + __shfl_xor(up ? p8[j] : p8[j + 4], 4, 64);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const bool up = r & 2;
+      p2[j] = (up ? p4[j + 2] : p4[j]) + __shfl_xor(up ? p4[j] : p4[j + 2], 2, 64);
+    }
+    const bool up1 = r & 1;
+    const float mine = ((up1 ? p2[1] : p2[0]) + __shfl_xor(up1 ? p2[0] : p2[1], 1, 64)) * qscale;
+    if (r < cnt && c_ok) o[(long)(row0 + ch * GLA_TC + r) * (H * Dv) + (long)h * Dv + c] = mine;
     if (ch + 1 < nch) stash(lds + ((ch + 1) & 1) * chunk);
     __syncthreads();
   }
   if (c_ok) {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-      const int d = r + 16 * i;
+      const int d = r * NR + i;
       if (d < D) sp[(long)d * Dv] = S[i];
     }
   }

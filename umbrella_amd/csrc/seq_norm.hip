@@ -50,7 +50,9 @@ __global__ __launch_bounds__(256) void embed_norm_kernel(float* __restrict__ x, 
   for (int i = lane; i < gs; i += 64) stf<P>(h + o + i, ldf<P>(er + i) * f * ldf<P>(w + grp * gs + i));
 }
 
-template <typename P>
+// values of one (row, group) held by a wave: lane owns elements lane + 64 j.  RV = 0: the group is longer than the register
+// budget and is re-read from memory in every pass.
+template <typename P, int RV>
 __global__ __launch_bounds__(256) void resid_norm_kernel(float* __restrict__ x, typename El<P>::type* __restrict__ h,
                                                          const float* __restrict__ y, const typename El<P>::type* __restrict__ w_post,
                                                          const typename El<P>::type* __restrict__ w_next, int W, int groups,
@@ -60,20 +62,53 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(float* __restrict__ x, 
   if (grp >= groups) return;
   const int t = blockIdx.x, gs = W / groups;
   const long o = (long)t * W + (long)grp * gs;
-  float ss = 0.f;
-  for (int i = lane; i < gs; i += 64) { const float v = y[o + i]; ss += v * v; }
-  ss = wave_sum(ss);
-  const float f = 1.f / sqrtf(ss / (float)gs + eps);
-  float s2 = 0.f;
-  for (int i = lane; i < gs; i += 64) {
-    const float v = x[o + i] + y[o + i] * f * ldf<P>(w_post + grp * gs + i);
-    x[o + i] = v;
-    s2 += v * v;
+  if constexpr (RV > 0) {
+    // all loads of the pass are issued before the first use: one memory round trip per pass instead of one per element
+    float yv[RV], xv[RV], wp[RV], wn[RV];
+#pragma unroll
+    for (int j = 0; j < RV; ++j) {
+      const int i = lane + 64 * j, ic = i < gs ? i : gs - 1;
+      yv[j] = y[o + ic];
+      xv[j] = x[o + ic];
+      wp[j] = ldf<P>(w_post + grp * gs + ic);
+      wn[j] = w_next ? ldf<P>(w_next + grp * gs + ic) : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < RV; ++j) ss += lane + 64 * j < gs ? yv[j] * yv[j] : 0.f;
+    ss = wave_sum(ss);
+    const float f = 1.f / sqrtf(ss / (float)gs + eps);
+    float s2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < RV; ++j) {
+      const int i = lane + 64 * j;
+      xv[j] = xv[j] + yv[j] * f * wp[j];
+      if (i < gs) { x[o + i] = xv[j]; s2 += xv[j] * xv[j]; }
+    }
+    if (!w_next) return;
+    s2 = wave_sum(s2);
+    const float f2 = 1.f / sqrtf(s2 / (float)gs + eps);
+#pragma unroll
+    for (int j = 0; j < RV; ++j) {
+      const int i = lane + 64 * j;
+      if (i < gs) stf<P>(h + o + i, xv[j] * f2 * wn[j]);
+    }
+  } else {
+    float ss = 0.f;
+    for (int i = lane; i < gs; i += 64) { const float v = y[o + i]; ss += v * v; }
+    ss = wave_sum(ss);
+    const float f = 1.f / sqrtf(ss / (float)gs + eps);
+    float s2 = 0.f;
+    for (int i = lane; i < gs; i += 64) {
+      const float v = x[o + i] + y[o + i] * f * ldf<P>(w_post + grp * gs + i);
+      x[o + i] = v;
+      s2 += v * v;
+    }
+    if (!w_next) return;
+    s2 = wave_sum(s2);
+    const float f2 = 1.f / sqrtf(s2 / (float)gs + eps);
+    for (int i = lane; i < gs; i += 64) stf<P>(h + o + i, x[o + i] * f2 * ldf<P>(w_next + grp * gs + i));
   }
-  if (!w_next) return;
-  s2 = wave_sum(s2);
-  const float f2 = 1.f / sqrtf(s2 / (float)gs + eps);
-  for (int i = lane; i < gs; i += 64) stf<P>(h + o + i, x[o + i] * f2 * ldf<P>(w_next + grp * gs + i));
 }
 
 static inline bool norm_args_ok(int T, int W, int groups) { return T >= 1 && W >= 1 && groups >= 1 && W % groups == 0; }
@@ -107,8 +142,17 @@ extern "C" int umb_seq_resid_norm(float* x, void* h, const float* y, const void*
   if (!norm_args_ok(T, W, groups) || !x || !y || !w_post || (w_next && !h)) return UMB_EINVAL;
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
-    hipLaunchKernelGGL(resid_norm_kernel<P>, dim3(T, (groups + 3) / 4), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
-                       (const E*)w_next, W, groups, eps);
+    const int per_lane = (W / groups + 63) / 64;
+    const dim3 grid(T, (groups + 3) / 4);
+    if (per_lane <= 4)
+      hipLaunchKernelGGL((resid_norm_kernel<P, 4>), grid, dim3(256), 0, st, x, (E*)h, y, (const E*)w_post, (const E*)w_next, W,
+                         groups, eps);
+    else if (per_lane <= 16)
+      hipLaunchKernelGGL((resid_norm_kernel<P, 16>), grid, dim3(256), 0, st, x, (E*)h, y, (const E*)w_post, (const E*)w_next, W,
+                         groups, eps);
+    else
+      hipLaunchKernelGGL((resid_norm_kernel<P, 0>), grid, dim3(256), 0, st, x, (E*)h, y, (const E*)w_post, (const E*)w_next, W,
+                         groups, eps);
   })
   UMB_LAUNCH_CHECK();
   return UMB_OK;

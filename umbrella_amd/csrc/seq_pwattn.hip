@@ -105,15 +105,16 @@ __global__ __launch_bounds__(64) void pwa_pool_kernel(UmbPagedKV kv, const int* 
 }
 
 // ---- attention.  Workgroup = (token, RH query heads of one key/value group): the heads of a group read the same keys and
-// values, so one pass over the keys serves all of them.  The four waves take the 64-key rounds w, w + 4, ... of the key list
+// values, so one pass over the keys serves all of them.  The NW waves take the 64-key rounds w, w + NW, ... of the key list
 // (pooled blocks first, then the window's tokens, both in position order) and their partial sums are added through LDS in
 // wave order -- which keys land in which wave depends on the query's position alone, never on the batch or on how the prompt
 // was cut.  Score phase: lane = key, 16-byte loads along the key's row against the queries held in LDS.  Value phase:
 // lane = value column, the round's weights broadcast one key at a time.
 constexpr int PWA_MAXC = 4;      // value columns per lane: D <= 256
+constexpr int PWA_KB = 8;        // keys whose value loads are in flight together
 
-template <typename P, int RH>
-__global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* __restrict__ out, const float* __restrict__ q,
+template <typename P, int RH, int NC, int NW>
+__global__ __launch_bounds__(NW * 64) void pwa_attend_kernel(typename El<P>::type* __restrict__ out, const float* __restrict__ q,
                                                          UmbPagedKV kv, const float* __restrict__ proj, int ld, int gate_col,
                                                          const typename El<P>::type* __restrict__ pos_bias,
                                                          const int* __restrict__ pos, const int* __restrict__ slot_, int T, int H,
@@ -122,13 +123,13 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* _
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int Dp = (D + 3) & ~3;
-  float* q_s = lds;                                          // [RH][Dp] queries; later [4][RH][Dp] partial outputs
-  float* w_s = lds + 4 * RH * Dp + wave * (RH * 64 + 128);   // per wave: [RH][64] weights, [64] 64-bit offsets
+  float* q_s = lds;                                          // [RH][Dp] queries; later [NW][RH][Dp] partial outputs
+  float* w_s = lds + NW * RH * Dp + wave * (RH * 64 + 128);  // per wave: [RH][64] weights, [64] 64-bit offsets
   long* off_s = reinterpret_cast<long*>(w_s + RH * 64);
   const int t = blockIdx.x, h0 = blockIdx.y * RH;
   const int g = h0 / (H / G);
   const int i = pos[t], slot = slot_[t];
-  for (int x = threadIdx.x; x < RH * D; x += 256) q_s[(x / D) * Dp + x % D] = q[(long)t * H * D + (long)h0 * D + x];
+  for (int x = threadIdx.x; x < RH * D; x += NW * 64) q_s[(x / D) * Dp + x % D] = q[(long)t * H * D + (long)h0 * D + x];
   float bias[RH];
 #pragma unroll
   for (int r = 0; r < RH; ++r) bias[r] = pos_bias ? ldf<P>(pos_bias + h0 + r) : 0.f;
@@ -137,12 +138,12 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* _
   const int n_blk = i - window + 1 >= pool ? (i - window + 1) / pool : 0;
   const int n_keys = n_blk + (i - j_lo + 1);
   const bool vec = (D & 7) == 0;
-  float acc[RH][PWA_MAXC];
+  float acc[RH][NC];
 #pragma unroll
   for (int r = 0; r < RH; ++r)
 #pragma unroll
-    for (int c = 0; c < PWA_MAXC; ++c) acc[r][c] = 0.f;
-  for (int base = wave * 64; base < n_keys; base += 256) {
+    for (int c = 0; c < NC; ++c) acc[r][c] = 0.f;
+  for (int base = wave * 64; base < n_keys; base += NW * 64) {
     const int kx = base + lane;
     float s[RH];
 #pragma unroll
@@ -154,23 +155,47 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* _
       off = pooled ? pkv_blk(kv, slot, kx, pool, g, G, D) : pkv_tok(kv, slot, j_lo + (kx - n_blk), g, G, D);
       if (pooled) {
         const float* kr = kv.kp + off;
-        for (int d = 0; d < D; ++d) {
-          const float kd = kr[d];
+        if ((D & 3) == 0) {
+          for (int d = 0; d < D; d += 32) {              // eight 16-byte loads in flight, then their 32 x RH products
+            f32x4 kk[8];
 #pragma unroll
-          for (int r = 0; r < RH; ++r) s[r] += q_s[r * Dp + d] * kd;
+            for (int u = 0; u < 8; ++u) kk[u] = *reinterpret_cast<const f32x4*>(kr + (d + 4 * u < D ? d + 4 * u : 0));
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              if (d + 4 * u >= D) break;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+#pragma unroll
+                for (int r = 0; r < RH; ++r) s[r] += q_s[r * Dp + d + 4 * u + e] * kk[u][e];
+              }
+            }
+          }
+        } else {
+          for (int d = 0; d < D; ++d) {
+            const float kd = kr[d];
+#pragma unroll
+            for (int r = 0; r < RH; ++r) s[r] += q_s[r * Dp + d] * kd;
+          }
         }
       } else {
         const E* kr = reinterpret_cast<const E*>(kv.k) + off;
         bool done = false;
         if constexpr (sizeof(E) == 2) {
           if (vec) {
-            for (int d = 0; d < D; d += 8) {
-              const u32x4 kk = *reinterpret_cast<const u32x4*>(kr + d);
+            for (int d = 0; d < D; d += 64) {            // eight 16-byte loads in flight, then their 64 x RH products
+              u32x4 kk[8];
 #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const float k0 = lo_f<P>(kk[e]), k1 = hi_f<P>(kk[e]);
+              for (int u = 0; u < 8; ++u) kk[u] = *reinterpret_cast<const u32x4*>(kr + (d + 8 * u < D ? d + 8 * u : 0));
 #pragma unroll
-                for (int r = 0; r < RH; ++r) s[r] += q_s[r * Dp + d + 2 * e] * k0 + q_s[r * Dp + d + 2 * e + 1] * k1;
+              for (int u = 0; u < 8; ++u) {
+                if (d + 8 * u >= D) break;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  const float k0 = lo_f<P>(kk[u][e]), k1 = hi_f<P>(kk[u][e]);
+                  const int dd = d + 8 * u + 2 * e;
+#pragma unroll
+                  for (int r = 0; r < RH; ++r) s[r] += q_s[r * Dp + dd] * k0 + q_s[r * Dp + dd + 1] * k1;
+                }
               }
             }
             done = true;
@@ -191,19 +216,47 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* _
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
     const int cnt = n_keys - base < 64 ? n_keys - base : 64;
-    for (int jj = 0; jj < cnt; ++jj) {
-      const long oj = off_s[jj];
-      float vv[PWA_MAXC];
+    // value rows: PWA_KB keys are fetched together, then used.  The round's keys are pooled entries first (fp32), then
+    // tokens (storage dtype): two loops, so that no load sits behind a branch on the entry's kind; indices past the end are
+    // clamped and weighted 0.
+    const int cntp = n_blk - base < 0 ? 0 : (n_blk - base < cnt ? n_blk - base : cnt);
+    int dcl[NC];
 #pragma unroll
-      for (int c = 0; c < PWA_MAXC; ++c) {
-        const int d = lane + 64 * c;
-        vv[c] = d < D ? (oj < 0 ? kv.vp[~oj + d] : ldf<P>(reinterpret_cast<const E*>(kv.v) + oj + d)) : 0.f;
+    for (int c = 0; c < NC; ++c) dcl[c] = lane + 64 * c < D ? lane + 64 * c : D - 1;
+    for (int j0 = 0; j0 < cntp; j0 += PWA_KB) {
+      float vv[PWA_KB][NC];
+#pragma unroll
+      for (int u = 0; u < PWA_KB; ++u) {
+        const long oj = ~off_s[j0 + u < cntp ? j0 + u : cntp - 1];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) vv[u][c] = kv.vp[oj + dcl[c]];
       }
 #pragma unroll
-      for (int r = 0; r < RH; ++r) {
-        const float wj = w_s[r * 64 + jj];
+      for (int u = 0; u < PWA_KB; ++u) {
 #pragma unroll
-        for (int c = 0; c < PWA_MAXC; ++c) acc[r][c] += wj * vv[c];
+        for (int r = 0; r < RH; ++r) {
+          const float wj = j0 + u < cntp ? w_s[r * 64 + j0 + u] : 0.f;
+#pragma unroll
+          for (int c = 0; c < NC; ++c) acc[r][c] += wj * vv[u][c];
+        }
+      }
+    }
+    for (int j0 = cntp; j0 < cnt; j0 += PWA_KB) {
+      float vv[PWA_KB][NC];
+#pragma unroll
+      for (int u = 0; u < PWA_KB; ++u) {
+        const long oj = off_s[j0 + u < cnt ? j0 + u : cnt - 1];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) vv[u][c] = ldf<P>(reinterpret_cast<const E*>(kv.v) + oj + dcl[c]);
+      }
+#pragma unroll
+      for (int u = 0; u < PWA_KB; ++u) {
+#pragma unroll
+        for (int r = 0; r < RH; ++r) {
+          const float wj = j0 + u < cnt ? w_s[r * 64 + j0 + u] : 0.f;
+#pragma unroll
+          for (int c = 0; c < NC; ++c) acc[r][c] += wj * vv[u][c];
+        }
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
@@ -213,16 +266,16 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(typename El<P>::type* _
 #pragma unroll
   for (int r = 0; r < RH; ++r)
 #pragma unroll
-    for (int c = 0; c < PWA_MAXC; ++c) {
+    for (int c = 0; c < NC; ++c) {
       const int d = lane + 64 * c;
       if (d < D) lds[(wave * RH + r) * Dp + d] = acc[r][c];
     }
   __syncthreads();
-  for (int x = threadIdx.x; x < RH * D; x += 256) {
+  for (int x = threadIdx.x; x < RH * D; x += NW * 64) {
     const int r = x / D, d = x % D;
     float o = lds[(0 * RH + r) * Dp + d];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) o += lds[(w * RH + r) * Dp + d];
+    for (int w = 1; w < NW; ++w) o += lds[(w * RH + r) * Dp + d];
     const float gate = 1.f / (1.f + expf(-proj[(long)t * ld + gate_col + h0 + r]));
     stf<P>(out + (long)t * H * D + (long)(h0 + r) * D + d, o * gate);
   }
@@ -266,18 +319,27 @@ extern "C" int umb_pwa_attend(void* out, const float* q, const UmbPagedKV* kv, c
   const int R = H / G;
   const int rh = R % 8 == 0 ? 8 : (R % 4 == 0 ? 4 : (R % 2 == 0 ? 2 : 1));     // heads of one group per workgroup
   const int Dp = (D + 3) & ~3;
-  const size_t lds = ((size_t)4 * rh * Dp + 4 * (rh * 64 + 128)) * sizeof(float);
   const dim3 grid(T, H / rh);
+  // few workgroups (decoding): sixteen waves share a query's keys, so a step's latency is one or two rounds; many (prompts):
+  // four, the chip is full anyway.  The choice changes the order in which a query's partial sums are added, nothing else.
+  const int nw = (long)T * (H / rh) < 1024 ? 16 : 4;
+  const size_t lds = ((size_t)nw * rh * Dp + nw * (rh * 64 + 128)) * sizeof(float);
+#define PWA_LAUNCH(RH, NC, NW)                                                                                            \
+  hipLaunchKernelGGL((pwa_attend_kernel<P, RH, NC, NW>), grid, dim3(NW * 64), lds, st, (E*)out, q, *kv, proj, ld, gate_col, \
+                     (const E*)pos_bias, pos, slot, T, H, G, D, window, pool, scale)
+#define PWA_NC(RH, NW)                                                                                                    \
+  if (D <= 64) PWA_LAUNCH(RH, 1, NW); else if (D <= 128) PWA_LAUNCH(RH, 2, NW); else PWA_LAUNCH(RH, 4, NW)
 #define PWA_CASE(RH)                                                                                                       \
   case RH:                                                                                                                 \
-    hipLaunchKernelGGL((pwa_attend_kernel<P, RH>), grid, dim3(256), lds, st, (E*)out, q, *kv, proj, ld, gate_col,          \
-                       (const E*)pos_bias, pos, slot, T, H, G, D, window, pool, scale);                                    \
+    if (nw == 16) { PWA_NC(RH, 16); } else { PWA_NC(RH, 4); }                                                              \
     break;
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
     switch (rh) { PWA_CASE(8) PWA_CASE(4) PWA_CASE(2) default: PWA_CASE(1) }
   })
 #undef PWA_CASE
+#undef PWA_NC
+#undef PWA_LAUNCH
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }
