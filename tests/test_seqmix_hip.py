@@ -62,6 +62,34 @@ def test_linear_silu_mul_epilogue(lib, dtype):
     assert ((out.cpu().double() - want).abs() <= rel * want.abs() + 1e-4).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,N,K", [(300, 200, 264), (257, 130, 72), (512, 256, 128)])
+def test_linear_many_tokens_tiled_through_lds(lib, dtype, T, N, K):
+    """prompts of >= 256 tokens take the 128 x 128 LDS-tiled kernel: ragged edges in all three dimensions, bias, the
+    rounding epilogue and the gate/up epilogue"""
+    from umbrella_amd import _lib
+    g = torch.Generator().manual_seed(T + N + K)
+    x, w, b = (torch.randn(s, generator=g).to(dtype) for s in ((T, K), (N, K), (N,)))
+    code = _lib.seq_dtype_code(dtype)
+    want = x.double() @ w.double().T + b.double()
+    out = torch.empty(T, N, dtype=torch.float32, device="cuda:0")
+    _lib.seq_call("umb_seq_linear", out, dev(x), dev(w), dev(b), T, N, K, 0, code)
+    assert (out.cpu().double() - want).abs().max() < 1e-4 * K ** 0.5
+    out_dt = torch.empty(T, N, dtype=dtype, device="cuda:0")
+    _lib.seq_call("umb_seq_linear", out_dt, dev(x), dev(w), dev(b), T, N, K, 1, code)
+    assert ((out_dt.cpu().double() - want).abs() <= 2.0 ** -8 * want.abs() + 1e-4 * K ** 0.5).all()
+    w2 = (0.2 * torch.randn(2 * N, K, generator=g)).to(dtype)
+    gate, up = x.double() @ w2[:N].double().T, x.double() @ w2[N:].double().T
+    act = torch.empty(T, N, dtype=dtype, device="cuda:0")
+    _lib.seq_call("umb_seq_linear", act, dev(x), dev(w2), None, T, 2 * N, K, 2, code)
+    want_act = gate * torch.sigmoid(gate) * up
+    assert ((act.cpu().double() - want_act).abs() <= 2.0 ** -8 * want_act.abs() + 1e-4 * K ** 0.5).all()
+    # the same rows through the skinny kernel (<= 64 tokens): equal up to the order of the fp32 sums
+    few = torch.empty(40, N, dtype=torch.float32, device="cuda:0")
+    _lib.seq_call("umb_seq_linear", few, dev(x[100:140]), dev(w), dev(b), 40, N, K, 0, code)
+    assert (few - out[100:140]).abs().max() < 1e-4 * K ** 0.5
+
+
 def test_linear_rows_do_not_depend_on_the_batch(lib):
     """a row's result is bit-identical whether it is computed alone, in a tile of 16 or among 70 rows"""
     from umbrella_amd import _lib

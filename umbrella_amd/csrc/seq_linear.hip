@@ -163,6 +163,127 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
   }
 }
 
+// ---- many tokens (T > 64), 16-bit storage: a 128 x 128 output tile per workgroup, operands staged through LDS.
+// The skinny kernel above streams every weight once per 64 tokens and every token fragment once per 16 (or 64) output rows
+// straight from L2: right when weights dominate, wasteful when both operands are re-used 128 times.  Here a stage of 64 k
+// (A: 128 output rows, B: 128 tokens, 16 KiB each) is fetched with 16-byte loads into registers while the previous stage is
+// consumed, written to the other half of a double-buffered 64 KiB LDS tile, and each of the four waves (2 x 2) reads the
+// fragments of its 64 x 64 sub-tile from there: 8 fragment reads per 16 MFMAs, every read a contiguous KiB (the tile is
+// stored as two [128 rows][32 k] halves so that a fragment's 16 rows x 64 B are adjacent: no bank conflict).
+// K is summed in order inside one accumulator (no K split): results differ from the skinny kernel by rounding only.
+// DUAL (gate/up): the 128 staged weight rows are 64 gate rows and the 64 up rows of the same outputs.
+template <typename P, bool DUAL>
+__global__ __launch_bounds__(256) void seq_linear_wide_kernel(void* __restrict__ out_, const u16* __restrict__ x,
+                                                              const u16* __restrict__ w, const u16* __restrict__ bias, int T,
+                                                              int N, int K, int epi) {
+  __shared__ __attribute__((aligned(16))) u16 tile[2][2][2][128 * 32];      // [buffer][A | B][k half][row][32 k]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int n0 = blockIdx.x * (DUAL ? 64 : 128), t0 = blockIdx.y * 128;
+  // staging: thread owns chunks c = tid + 256 i (i < 4) of each operand's 128 x 8 chunk grid: row c / 8, 16-byte chunk c % 8
+  const u16* asrc[4];
+  const u16* bsrc[4];
+  bool aok[4], bok[4];
+  int soff[4], kc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = tid + 256 * i, row = c >> 3, ch = c & 7;
+    int n = DUAL ? (row < 64 ? n0 + row : N + n0 + (row - 64)) : n0 + row;
+    aok[i] = DUAL ? (n0 + (row & 63) < N) : (n < N);
+    asrc[i] = w + (long)(aok[i] ? n : 0) * K + ch * 8;
+    bok[i] = t0 + row < T;
+    bsrc[i] = x + (long)(bok[i] ? t0 + row : 0) * K + ch * 8;
+    kc[i] = ch * 8;
+    soff[i] = (ch >> 2) * (128 * 32) + row * 32 + (ch & 3) * 8;
+  }
+  u32x4 ra[4], rb[4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool in = k0 + kc[i] < K;
+      ra[i] = (aok[i] && in) ? *reinterpret_cast<const u32x4*>(asrc[i] + k0) : u32x4{0u, 0u, 0u, 0u};
+      rb[i] = (bok[i] && in) ? *reinterpret_cast<const u32x4*>(bsrc[i] + k0) : u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<u32x4*>(&tile[buf][0][0][0] + soff[i]) = ra[i];
+      *reinterpret_cast<u32x4*>(&tile[buf][1][0][0] + soff[i]) = rb[i];
+    }
+  };
+  int arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) arow[i] = DUAL ? ((i >> 1) * 64 + wm * 32 + (i & 1) * 16) : (wm * 64 + i * 16);
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) acc[i][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int nst = (K + 63) / 64;
+  for (int st = 0; st < nst; ++st) {
+    const int buf = st & 1;
+    if (st + 1 < nst) fetch((st + 1) * 64);
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      u32x4 fa[4], fb[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        fa[i] = *reinterpret_cast<const u32x4*>(&tile[buf][0][kh][(arow[i] + j) * 32 + g * 8]);
+        fb[i] = *reinterpret_cast<const u32x4*>(&tile[buf][1][kh][(wn * 64 + i * 16 + j) * 32 + g * 8]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) acc[i][tt] = P::mfma(fa[i], fb[tt], acc[i][tt]);
+    }
+    if (st + 1 < nst) stash(buf ^ 1);
+    __syncthreads();
+  }
+  // lane holds outputs (row = 4 g + r of its A tile, token = j of its B tile)
+#pragma unroll
+  for (int tt = 0; tt < 4; ++tt) {
+    const int t = t0 + wn * 64 + tt * 16 + j;
+    if (t >= T) continue;
+#pragma unroll
+    for (int i = 0; i < (DUAL ? 2 : 4); ++i) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = n0 + (DUAL ? wm * 32 + i * 16 : arow[i]) + 4 * g + r;
+        if (n >= N) continue;
+        float sv = acc[i][tt][r] + (bias ? P::to_f(bias[n]) : 0.f);
+        if constexpr (DUAL) {
+          const float uv = acc[i + 2][tt][r] + (bias ? P::to_f(bias[N + n]) : 0.f);
+          reinterpret_cast<u16*>(out_)[(long)t * N + n] = P::from_f(siluf_(sv) * uv);
+        } else if (epi == EPI_DT) {
+          reinterpret_cast<u16*>(out_)[(long)t * N + n] = P::from_f(sv);
+        } else {
+          reinterpret_cast<float*>(out_)[(long)t * N + n] = sv;
+        }
+      }
+    }
+  }
+}
+
+template <typename P>
+static int launch_wide(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st) {
+  if constexpr (sizeof(typename El<P>::type) == 2) {
+    if (epi == EPI_SILU_MUL)
+      hipLaunchKernelGGL((seq_linear_wide_kernel<P, true>), dim3((N + 63) / 64, (T + 127) / 128), dim3(256), 0, st, out,
+                         (const u16*)x, (const u16*)w, (const u16*)bias, T, N, K, epi);
+    else
+      hipLaunchKernelGGL((seq_linear_wide_kernel<P, false>), dim3((N + 127) / 128, (T + 127) / 128), dim3(256), 0, st, out,
+                         (const u16*)x, (const u16*)w, (const u16*)bias, T, N, K, epi);
+    UMB_LAUNCH_CHECK();
+    return UMB_OK;
+  } else {
+    return UMB_EINVAL;
+  }
+}
+
 template <typename P, int NT, int TT, bool VEC>
 static int launch_tt(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st) {
   typedef typename El<P>::type E;
@@ -184,8 +305,10 @@ static int launch_vec(void* out, const void* x, const void* w, const void* bias,
   if (T <= 32) return launch_tt<P, 1, 2, VEC>(out, x, w, bias, T, N, K, epi, st);
   // many tokens: the launch is bound by fragment loads per MFMA, not by weight bytes -> four output tiles per workgroup
   // (the K order of every output is unchanged: a row's value does not depend on which variant computed it)
-  if (T > 64 && N >= 64 && sizeof(typename El<P>::type) == 2)
+  if (T > 64 && N >= 64 && sizeof(typename El<P>::type) == 2) {
+    if (VEC && T >= 256 && N >= 128) return launch_wide<P>(out, x, w, bias, T, N, K, epi, st);      // both operands re-used
     return launch_tt<P, 4, 4, VEC>(out, x, w, bias, T, N, K, epi, st);
+  }
   return launch_tt<P, 1, 4, VEC>(out, x, w, bias, T, N, K, epi, st);
 }
 
