@@ -84,6 +84,14 @@ int umb_pwa_attend(void* out, const float* q, const UmbPagedKV* kv, const float*
                    const int* pos, const int* slot, int T, int H, int G, int D, int window, int pool, float scale, int dtype,
                    umb_stream_t stream);
 
+/* The same attention for steps that bring whole stretches of a sequence (prompts), on the matrix pipe: 16-bit storage only,
+ * D a multiple of 32 (<= 256); workgroups own 16 consecutive positions of one sequence.  Scores and weights keep fp32
+ * accuracy: the fp32 factors (q, pooled means, weights) enter as high + low 16-bit halves. */
+int umb_pwa_attend_tiled(void* out, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
+                         const void* pos_bias, const int* seq_slot, const int* seq_row0, const int* seq_pos0, const int* seq_len,
+                         int B, int max_len, int H, int G, int D, int window, int pool, float scale, int dtype,
+                         umb_stream_t stream);
+
 /* ------------------------------------------------------------------ the model */
 typedef struct UmbSeqLayer {
   int32_t kind, has_mlp;

@@ -214,7 +214,7 @@ def _attn_weights(width, H, G, D, seed):
                 wg=r(H, width) / width ** 0.5, wo=r(width, H * D) / (H * D) ** 0.5, bo=0.1 * r(width), pb=0.5 * r(H))
 
 
-def _run_attn(X, w, H, G, D, window, pool, rot_dims, base, scale, eps, dtype, page, splits, seq="s", cache=None):
+def _run_attn(X, w, H, G, D, window, pool, rot_dims, base, scale, eps, dtype, page, splits, seq="s", cache=None, tiled=False):
     """the library's prep -> pool -> attend on the rows of X through a paged cache, cut into consecutive steps"""
     from umbrella_amd import _lib
     from umbrella_amd.attn.cache import PagedSeqCache
@@ -240,8 +240,13 @@ def _run_attn(X, w, H, G, D, window, pool, rot_dims, base, scale, eps, dtype, pa
         _lib.seq_call("umb_pwa_prep", q, kv, proj, ld, pos, slots, freq, n, H, G, D, rot_dims, eps, code)
         _lib.seq_call("umb_pwa_pool", kv, meta[0:1], meta[1:2], meta[2:3], 1, n, G, D, pool, code)
         mix = torch.empty(n, H * D, dtype=dtype, device="cuda:0")
-        _lib.seq_call("umb_pwa_attend", mix, q, kv, proj, ld, H * D + G * D, dev(w["pb"], dtype), pos, slots, n, H, G, D, window,
-                      pool, float(scale), code)
+        if tiled and n >= 16:                # as the model does: stretches of a sequence go to the matrix-pipe kernel
+            one = torch.tensor([0], dtype=torch.int32, device="cuda:0")
+            _lib.seq_call("umb_pwa_attend_tiled", mix, q, kv, proj, ld, H * D + G * D, dev(w["pb"], dtype), meta[0:1], one,
+                          meta[1:2], meta[2:3], 1, n, H, G, D, window, pool, float(scale), code)
+        else:
+            _lib.seq_call("umb_pwa_attend", mix, q, kv, proj, ld, H * D + G * D, dev(w["pb"], dtype), pos, slots, n, H, G, D,
+                          window, pool, float(scale), code)
         y = torch.empty(n, width, dtype=torch.float32, device="cuda:0")
         _lib.seq_call("umb_seq_linear", y, mix, dev(w["wo"], dtype), dev(w["bo"], dtype), n, width, H * D, 0, code)
         outs.append(y)
@@ -311,6 +316,42 @@ def test_attention_window_and_pool_edges_with_standout_keys(lib, dtype):
     for splits in ([n], [12] + [1] * (n - 12), [16] + [1] * (n - 16), [15] + [1] * (n - 15), [2] * (n // 2)):
         got, _ = _run_attn(X, w, dtype=dtype, page=page, splits=splits, **kw)
         assert (got.cpu().double() - want).abs().max() < tol, splits
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("H,G,D,window,pool,rot_dims,page", [(4, 2, 32, 6, 3, 32, 4), (8, 2, 64, 9, 7, 16, 5), (3, 3, 32, 1, 1, 8, 3),
+                                                             (2, 1, 96, 20, 4, 0, 64)])
+def test_attention_on_the_matrix_pipe(lib, dtype, H, G, D, window, pool, rot_dims, page):
+    """prompt stretches of >= 16 tokens through the MFMA kernel (every phase of window, block, page and 16-query tile),
+    against the oracle and against the vector-pipe kernel: the two must agree to the rounding of their 16-bit outputs"""
+    width, n, eps, base = 40, 70, 1e-5, 100.0
+    w = _attn_weights(width, H, G, D, seed=H + D)
+    X = torch.randn(n, width, generator=torch.Generator().manual_seed(11))
+    kw = dict(H=H, G=G, D=D, window=window, pool=pool, rot_dims=rot_dims, base=base, scale=0.21, eps=eps)
+    want = _attn_oracle(X, w, dtype, **kw)
+    plain, _ = _run_attn(X, w, dtype=dtype, page=page, splits=[n], **kw)
+    # the mixer output is rounded to the storage dtype before the output projection: errors scale with the outputs
+    tol = (1.2e-2 if dtype == torch.bfloat16 else 2e-3) * max(1.0, float(want.abs().max()))
+    assert (plain.cpu().double() - want).abs().max() < tol
+    for splits in ([n], [33, 37], [16, 16, 16, 16, 6], [20] + [1] * 50, [17, 1, 1, 18, 33]):
+        got, _ = _run_attn(X, w, dtype=dtype, page=page, splits=splits, tiled=True, **kw)
+        assert (got.cpu().double() - want).abs().max() < tol, splits
+        assert (got - plain).abs().max() < tol / 2, splits
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_matrix_pipe_window_and_pool_edges_with_standout_keys(lib, dtype):
+    """the counting test of the vector-pipe kernel, on the MFMA kernel: tiles of 16 queries that straddle every edge"""
+    H, G, D, window, pool, page, width, n, eps = 2, 1, 32, 5, 4, 3, 16, 48, 1e-6
+    loud = [8, 9, 10, 11]
+    w, X = _standout(n, width, H, G, D, loud)
+    kw = dict(H=H, G=G, D=D, window=window, pool=pool, rot_dims=0, base=10.0, scale=12.0 / D, eps=eps)
+    want = _attn_oracle(X, w, dtype, **kw)
+    count = (want[:, 0] / 0.25).round().int().tolist()
+    assert count[7:17] == [0, 1, 2, 3, 4, 4, 3, 2, 1, 1] and count[17:] == [1] * (n - 17)
+    for splits in ([n], [16, 32], [24, 24], [17, 31]):
+        got, _ = _run_attn(X, w, dtype=dtype, page=page, splits=splits, tiled=True, **kw)
+        assert (got.cpu().double() - want).abs().max() < 2e-2, splits
 
 
 def test_attention_pages_are_reused_without_leaking(lib):

@@ -253,6 +253,7 @@ SEQ_SIGNATURES = {
     "umb_pwa_prep": [_P, _PKV, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I],
     "umb_pwa_pool": [_PKV, _P, _P, _P, _I, _I, _I, _I, _I, _I],
     "umb_pwa_attend": [_P, _P, _PKV, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I],
+    "umb_pwa_attend_tiled": [_P, _P, _PKV, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I],
     "umb_seq_forward": [C.POINTER(UmbSeqModel), C.POINTER(UmbSeqWork), C.POINTER(UmbSeqStep)],
     "umb_argmax_rows": [_P, _P, _I, _I],
     "umb_sample_rows": [_P, _P, _I, _I, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P],

@@ -11,6 +11,7 @@
 // sequence was cut into steps.  The token loop is the only serial dimension; its inputs are independent of the recurrence and
 // are staged ahead through LDS in chunks of 16 tokens.
 #include "seq_common.h"
+#include <type_traits>
 
 template <typename P>
 __global__ __launch_bounds__(256) void gla_decay_kernel(float* __restrict__ alpha, const float* __restrict__ proj, int ld,
@@ -37,14 +38,17 @@ constexpr int GLA_COLS = 16;     // value columns per workgroup (4 per wave)
 // Workgroup = (sequence, head, 16 value columns), 4 waves of 4 columns.  The token loop is serial, so its inputs must not
 // cost a memory round trip per token: chunks of 16 tokens (alpha, k, q rows of the head and the 16 v columns) are staged
 // through a double-buffered LDS tile -- the global loads of chunk c + 1 are in flight while chunk c is consumed from LDS.
-template <int NR>
+// V4: D, Dv and the row stride of proj are multiples of 4 -> the staging moves 16-byte pieces (a quarter of the address
+// arithmetic, which is what this issue-bound kernel spends its time on).
+template <int NR, bool V4>
 __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, float* __restrict__ state,
                                                        const float* __restrict__ proj, int ld, const float* __restrict__ alpha,
                                                        const int* __restrict__ seq_slot, const int* __restrict__ seq_row0,
                                                        const int* __restrict__ seq_pos0, const int* __restrict__ seq_len, int H,
                                                        int D, int Dv, float qscale) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int STG = 3 * NR + 1;                       // staged elements per thread: TC (3 D + 16) / 256 <= 3 NR + 1
+  constexpr int VW = V4 ? 4 : 1;                        // floats per staged piece
+  constexpr int STG = (3 * NR + 1 + VW - 1) / VW;       // staged pieces per thread: TC (3 D + 16) / 256 <= 3 NR + 1 floats
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15;
   const int cbase = blockIdx.x * GLA_COLS, cl = wave * 4 + (lane >> 4), c = cbase + cl;
   const int h = blockIdx.y, b = blockIdx.z;
@@ -62,37 +66,39 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, fl
   }
   const int HD = H * D, rowlen = 3 * D + GLA_COLS, chunk = GLA_TC * rowlen;
   const int nch = (n + GLA_TC - 1) / GLA_TC;
-  float stage[STG];
+  typedef typename std::conditional<V4, f32x4, float>::type piece;
+  piece stage[STG];
+  const int rowp = rowlen / VW, chunkp = chunk / VW;    // in pieces
   // chunk ch -> registers.  Every load is unconditional and lands on a valid address (indices are clamped): loads that sit in
   // divergent branches would each wait for their own round trip.  What a clamped load brings is never used: tokens past the
   // sequence are not consumed, columns past Dv are not written, indices past the chunk are not stashed.
-  const int tt0 = tid / rowlen, ci0 = tid - tt0 * rowlen;
+  const int tt0 = tid / rowp, ci0 = (tid - tt0 * rowp) * VW;
   auto fetch = [&](int ch) {
-    int tt = tt0, ci = ci0;                             // (token, column) of staged element e * 256 + tid, kept incrementally
+    int tt = tt0, ci = ci0;                             // (token, column) of staged piece e * 256 + tid, kept incrementally
 #pragma unroll
     for (int e = 0; e < STG; ++e) {
       if (e) {
-        ci += 256;
+        ci += 256 * VW;
         while (ci >= rowlen) { ci -= rowlen; ++tt; }
-        if (tt >= GLA_TC) { tt = GLA_TC - 1; ci = rowlen - 1; }      // past the chunk: any valid address
+        if (tt >= GLA_TC) { tt = GLA_TC - 1; ci = rowlen - VW; }     // past the chunk: any valid address
       }
       int t = ch * GLA_TC + tt;
       t = t < n ? t : n - 1;
       const long row = row0 + t;
       int vc = cbase + ci - 3 * D;
-      vc = vc < Dv ? vc : Dv - 1;
+      vc = vc + VW <= Dv ? vc : Dv - VW;
       const float* src = ci < D ? alpha + row * HD + (long)h * D + ci
                        : ci < 2 * D ? proj + row * ld + HD + (long)h * D + (ci - D)
                        : ci < 3 * D ? proj + row * ld + (long)h * D + (ci - 2 * D)
                                     : proj + row * ld + 2L * HD + (long)h * Dv + vc;
-      stage[e] = *src;
+      stage[e] = *reinterpret_cast<const piece*>(src);
     }
   };
   auto stash = [&](float* buf) {
 #pragma unroll
     for (int e = 0; e < STG; ++e) {
       const int idx = e * 256 + tid;
-      if (idx < chunk) buf[idx] = stage[e];
+      if (idx < chunkp) reinterpret_cast<piece*>(buf)[idx] = stage[e];
     }
   };
   fetch(0);
@@ -213,13 +219,18 @@ extern "C" int umb_gla_scan(float* o, float* state, const float* proj, int ld, c
   const dim3 grid((Dv + GLA_COLS - 1) / GLA_COLS, H, B);
   const int nr = (D + 15) / 16;
   const size_t lds = 2 * (size_t)GLA_TC * (3 * D + GLA_COLS) * sizeof(float);
+  const bool v4 = D % 4 == 0 && Dv % 4 == 0 && ld % 4 == 0;
+#define GLA_SCAN_LAUNCH(NR, V4)                                                                                           \
+  do {                                                                                                                    \
+    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)gla_scan_kernel<NR, V4>,                                      \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)       \
+      return UMB_EHIP;                                                                                                    \
+    hipLaunchKernelGGL((gla_scan_kernel<NR, V4>), grid, dim3(256), lds, st, o, state, proj, ld, alpha, seq_slot, seq_row0, \
+                       seq_pos0, seq_len, H, D, Dv, qscale);                                                              \
+  } while (0)
 #define GLA_SCAN_CASE(NR)                                                                                                 \
   case NR:                                                                                                                \
-    if (lds > 48 * 1024 &&                                                                                                \
-        hipFuncSetAttribute((const void*)gla_scan_kernel<NR>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
-      return UMB_EHIP;                                                                                                    \
-    hipLaunchKernelGGL(gla_scan_kernel<NR>, grid, dim3(256), lds, st, o, state, proj, ld, alpha, seq_slot, seq_row0, seq_pos0, \
-                       seq_len, H, D, Dv, qscale);                                                                        \
+    if (v4) GLA_SCAN_LAUNCH(NR, true); else GLA_SCAN_LAUNCH(NR, false);                                                   \
     break;
   switch (nr) {
     GLA_SCAN_CASE(1) GLA_SCAN_CASE(2) GLA_SCAN_CASE(3) GLA_SCAN_CASE(4) GLA_SCAN_CASE(5) GLA_SCAN_CASE(6) GLA_SCAN_CASE(7)
@@ -228,6 +239,7 @@ extern "C" int umb_gla_scan(float* o, float* state, const float* proj, int ld, c
     default: return UMB_EINVAL;
   }
 #undef GLA_SCAN_CASE
+#undef GLA_SCAN_LAUNCH
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }

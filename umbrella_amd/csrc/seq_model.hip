@@ -3,7 +3,7 @@
 //     x <- x + norm1b(mixer(norm1(x)))      x <- x + norm2b(ff(norm2(x)))    (the second only where the layer has one)
 // with every norm a grouped RMS norm.  The seam kernel (resid_norm) adds a sublayer's normed output into the fp32 residual
 // stream and produces the next sublayer's normed input in one pass, so a layer is
-//     attention: proj GEMM | rope + unit-norm + append | pool | attend | out GEMM | seam | gate-up GEMM (SiLU*up epilogue) |
+//     attention: proj GEMM | rope + unit-norm + append | pool | attend (matrix pipe for prompts) | out GEMM | seam | gate-up GEMM (SiLU*up epilogue) |
 //                down GEMM | seam
 //     GLA:       proj GEMM | decay | scan | head norm * SiLU gate | out GEMM | seam (| feed-forward as above)
 // Nothing here depends on the host between launches: a step can be captured into a hipGraph.
@@ -36,8 +36,13 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
       if (ly.vdim != D || ld != H * D + G * D + H) return UMB_EINVAL;
       SEQ_TRY(umb_pwa_prep(ws->aux, &ly.kv, ws->proj, ld, s->pos, s->slot, ly.rot_freq, T, H, G, D, ly.rot_dims, eps, dt, st));
       SEQ_TRY(umb_pwa_pool(&ly.kv, s->seq_slot, s->seq_pos0, s->seq_len, s->B, s->max_len, G, D, ly.pool, dt, st));
-      SEQ_TRY(umb_pwa_attend(ws->mix, ws->aux, &ly.kv, ws->proj, ld, H * D + G * D, ly.pos_bias, s->pos, s->slot, T, H, G, D,
-                             ly.window, ly.pool, ly.scale, dt, st));
+      // steps that bring stretches of a sequence (prompts) take the matrix-pipe kernel where the shape allows it
+      if (dt != UMB_SEQ_F32 && D % 32 == 0 && D <= 256 && s->max_len >= 16)
+        SEQ_TRY(umb_pwa_attend_tiled(ws->mix, ws->aux, &ly.kv, ws->proj, ld, H * D + G * D, ly.pos_bias, s->seq_slot, s->seq_row0,
+                                     s->seq_pos0, s->seq_len, s->B, s->max_len, H, G, D, ly.window, ly.pool, ly.scale, dt, st));
+      else
+        SEQ_TRY(umb_pwa_attend(ws->mix, ws->aux, &ly.kv, ws->proj, ld, H * D + G * D, ly.pos_bias, s->pos, s->slot, T, H, G, D,
+                               ly.window, ly.pool, ly.scale, dt, st));
     } else if (ly.kind == UMB_MIX_GLA) {
       const int H = ly.heads, D = ly.dim, Dv = ly.vdim, HD = H * D;
       if (ld != 2 * HD + 2 * H * Dv + ly.rank || !ly.state) return UMB_EINVAL;

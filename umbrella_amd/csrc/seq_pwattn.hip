@@ -281,6 +281,185 @@ __global__ __launch_bounds__(NW * 64) void pwa_attend_kernel(typename El<P>::typ
   }
 }
 
+// ---- prompt attention on the matrix pipe (16-bit storage, D a multiple of 32).
+// Workgroup = (16 consecutive positions of one sequence, one key/value group); its four waves take the group's query heads.
+// Key list of the tile: pooled blocks 0 .. nb(last position) (padded to a multiple of 32), then the tokens from the first
+// position's window start to the last position; a 32-key step is all pooled or all tokens.  Per step and head:
+//   S^T = K Q^T as two 16-key MFMA tiles (A = 16 keys x 32 d straight from the cache rows, B = the queries);
+//   P = visible ? sigmoid(S scale + bias) : 0 in fp32, lane (query j, key quad g) holding keys 4g .. 4g+3 of both tiles --
+//   which IS the lane's share of the B operand of O^T += V^T P^T over the step's 32 keys when V^T's k index runs over
+//   (tile 0: 4g..4g+3, tile 1: 4g..4g+3): no data moves between the two products;
+//   V^T (A operand: 16 d x those 8 keys) is gathered from a [32 keys][D] copy of the value rows in LDS.
+// Scores and weights stay fp32-exact on a bf16 / f16 matrix pipe by splitting the fp32 factor into a high and a low 16-bit
+// half (x = hi + lo to 2^-17): q, the pooled means (held in fp32) and the weights go through two MFMAs instead of one.
+template <typename P> __device__ __forceinline__ void split8(const float* v, u32x4& hi, u32x4& lo) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const u16 h0 = P::from_f(v[2 * e]), h1 = P::from_f(v[2 * e + 1]);
+    const u16 l0 = P::from_f(v[2 * e] - P::to_f(h0)), l1 = P::from_f(v[2 * e + 1] - P::to_f(h1));
+    hi[e] = (unsigned)h0 | ((unsigned)h1 << 16);
+    lo[e] = (unsigned)l0 | ((unsigned)l1 << 16);
+  }
+}
+
+template <typename P, int NS>
+__global__ __launch_bounds__(256) void pwa_attend_mfma_kernel(u16* __restrict__ out, const float* __restrict__ q, UmbPagedKV kv,
+                                                              const float* __restrict__ proj, int ld, int gate_col,
+                                                              const u16* __restrict__ pos_bias, const int* __restrict__ seq_slot,
+                                                              const int* __restrict__ seq_row0, const int* __restrict__ seq_pos0,
+                                                              const int* __restrict__ seq_len, int H, int G, int window, int pool,
+                                                              float scale) {
+  constexpr int D = NS * 32, LD = D + 8;              // LDS row stride: 16 bytes of padding spread the key quads over the banks
+  extern __shared__ __attribute__((aligned(16))) u16 vt_all[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g4 = lane >> 4;
+  u16* v_hi = vt_all + (long)wave * (2 * 32 * LD + 32 * 4);   // [32][LD] values, [32][LD] low halves (pooled steps), [32] offsets
+  u16* v_lo = v_hi + 32 * LD;
+  long* offs = reinterpret_cast<long*>(v_lo + 32 * LD);
+  const int b = blockIdx.y, g = blockIdx.z;
+  const int n = seq_len[b], q0 = blockIdx.x * 16;
+  if (q0 >= n) return;
+  const int slot = seq_slot[b], row0 = seq_row0[b], pos0 = seq_pos0[b];
+  const int nq = n - q0 < 16 ? n - q0 : 16;
+  const int i_first = pos0 + q0, i_last = i_first + nq - 1;
+  const bool q_ok = j < nq;
+  const int i_j = i_first + (q_ok ? j : nq - 1);
+  const long qrow = row0 + q0 + (q_ok ? j : nq - 1);
+  const int nb_j = i_j - window + 1 >= pool ? (i_j - window + 1) / pool : 0;
+  const int nb_max = i_last - window + 1 >= pool ? (i_last - window + 1) / pool : 0;
+  const int j_lo = i_first - window + 1 > 0 ? i_first - window + 1 : 0;
+  const int tok0 = (nb_max + 31) & ~31, total = tok0 + (i_last - j_lo + 1);
+  const int R = H / G;
+  for (int r = wave; r < R; r += 4) {
+    const int h = g * R + r;
+    u32x4 qhi[NS], qlo[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      float v[8];
+      const f32x4 a = *reinterpret_cast<const f32x4*>(q + qrow * H * D + (long)h * D + 32 * s + 8 * g4);
+      const f32x4 c = *reinterpret_cast<const f32x4*>(q + qrow * H * D + (long)h * D + 32 * s + 8 * g4 + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { v[e] = a[e]; v[4 + e] = c[e]; }
+      split8<P>(v, qhi[s], qlo[s]);
+    }
+    const float bias = pos_bias ? P::to_f(pos_bias[h]) : 0.f;
+    f32x4 o[2 * NS];
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int base = 0; base < total; base += 32) {
+      const bool pooled = base < tok0;
+      // element offsets of the step's 32 keys (-1: no such key)
+      if (lane < 32) {
+        const int kx = base + lane;
+        long off = -1;
+        if (pooled) { if (kx < nb_max) off = pkv_blk(kv, slot, kx, pool, g, G, D); }
+        else if (kx < total) off = pkv_tok(kv, slot, j_lo + (kx - tok0), g, G, D);
+        offs[lane] = off;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      // value rows -> LDS: 32 x D / 8 pieces of 8 features, NS pieces... (4 D / 64 = 2 NS per lane)
+#pragma unroll
+      for (int i = 0; i < 2 * NS; ++i) {
+        const int p = lane + 64 * i, m = p / (D / 8), dp = (p % (D / 8)) * 8;
+        const long off = offs[m];
+        u32x4 hi = u32x4{0u, 0u, 0u, 0u}, lo = u32x4{0u, 0u, 0u, 0u};
+        if (off >= 0) {
+          if (pooled) {
+            float v[8];
+            const f32x4 a = *reinterpret_cast<const f32x4*>(kv.vp + off + dp);
+            const f32x4 c = *reinterpret_cast<const f32x4*>(kv.vp + off + dp + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[e] = a[e]; v[4 + e] = c[e]; }
+            split8<P>(v, hi, lo);
+          } else {
+            hi = *reinterpret_cast<const u32x4*>(reinterpret_cast<const u16*>(kv.v) + off + dp);
+          }
+        }
+        *reinterpret_cast<u32x4*>(v_hi + m * LD + dp) = hi;
+        if (pooled) *reinterpret_cast<u32x4*>(v_lo + m * LD + dp) = lo;
+      }
+      // scores of the two 16-key tiles
+      f32x4 sc[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        sc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const long off = offs[16 * u + j];
+        const long offc = off >= 0 ? off : 0;
+        if (pooled) {
+#pragma unroll
+          for (int s = 0; s < NS; ++s) {
+            float v[8];
+            const f32x4 a = *reinterpret_cast<const f32x4*>(kv.kp + offc + 32 * s + 8 * g4);
+            const f32x4 c = *reinterpret_cast<const f32x4*>(kv.kp + offc + 32 * s + 8 * g4 + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[e] = a[e]; v[4 + e] = c[e]; }
+            u32x4 khi, klo;
+            split8<P>(v, khi, klo);
+            sc[u] = P::mfma(khi, qhi[s], sc[u]);
+            sc[u] = P::mfma(khi, qlo[s], sc[u]);
+            sc[u] = P::mfma(klo, qhi[s], sc[u]);
+          }
+        } else {
+          u32x4 kf[NS];
+#pragma unroll
+          for (int s = 0; s < NS; ++s)
+            kf[s] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const u16*>(kv.k) + offc + 32 * s + 8 * g4);
+#pragma unroll
+          for (int s = 0; s < NS; ++s) {
+            sc[u] = P::mfma(kf[s], qhi[s], sc[u]);
+            sc[u] = P::mfma(kf[s], qlo[s], sc[u]);
+          }
+        }
+      }
+      // weights: lane (query j, quad g4) holds keys 16 u + 4 g4 + r of the step
+      float w[8];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int kk = base + 16 * u + 4 * g4 + rr;
+          bool vis;
+          if (pooled) vis = kk < nb_j;
+          else { const int jt = j_lo + (kk - tok0); vis = jt <= i_j && jt > i_j - window; }
+          w[4 * u + rr] = (vis && q_ok) ? 1.f / (1.f + expf(-(sc[u][rr] * scale + bias))) : 0.f;
+        }
+      u32x4 phi, plo;
+      split8<P>(w, phi, plo);
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      // O^T[d][query] += V^T[d][keys] P^T[keys][query]: lane (d row j of tile dt, quad g4) gathers its 8 keys' values
+#pragma unroll
+      for (int dt = 0; dt < 2 * NS; ++dt) {
+        unsigned e[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m) e[m] = v_hi[((m >> 2) * 16 + 4 * g4 + (m & 3)) * LD + 16 * dt + j];
+        const u32x4 va = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+        o[dt] = P::mfma(va, phi, o[dt]);
+        o[dt] = P::mfma(va, plo, o[dt]);
+        if (pooled) {
+#pragma unroll
+          for (int m = 0; m < 8; ++m) e[m] = v_lo[((m >> 2) * 16 + 4 * g4 + (m & 3)) * LD + 16 * dt + j];
+          const u32x4 vl = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+          o[dt] = P::mfma(vl, phi, o[dt]);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    // lane holds O^T[d = 16 dt + 4 g4 + rr][query j]
+    if (q_ok) {
+      const float gate = 1.f / (1.f + expf(-proj[qrow * ld + gate_col + h]));
+#pragma unroll
+      for (int dt = 0; dt < 2 * NS; ++dt) {
+        u32x2 pk;
+        pk[0] = pack2<P>(o[dt][0] * gate, o[dt][1] * gate);
+        pk[1] = pack2<P>(o[dt][2] * gate, o[dt][3] * gate);
+        *reinterpret_cast<u32x2*>(out + qrow * H * D + (long)h * D + 16 * dt + 4 * g4) = pk;
+      }
+    }
+  }
+}
+
 static inline bool pkv_ok(const UmbPagedKV* kv) {
   return kv && kv->k && kv->v && kv->kp && kv->vp && kv->pages && kv->page >= 1 && kv->max_pages >= 1;
 }
@@ -340,6 +519,39 @@ extern "C" int umb_pwa_attend(void* out, const float* q, const UmbPagedKV* kv, c
 #undef PWA_CASE
 #undef PWA_NC
 #undef PWA_LAUNCH
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_pwa_attend_tiled(void* out, const float* q, const UmbPagedKV* kv, const float* proj, int ld, int gate_col,
+                                    const void* pos_bias, const int* seq_slot, const int* seq_row0, const int* seq_pos0,
+                                    const int* seq_len, int B, int max_len, int H, int G, int D, int window, int pool, float scale,
+                                    int dtype, hipStream_t st) {
+  if (B < 1 || max_len < 1 || H < 1 || G < 1 || H % G || D < 32 || D > 256 || D % 32 || window < 1 || pool < 1 || !out || !q ||
+      !pkv_ok(kv) || !proj || !seq_slot || !seq_row0 || !seq_pos0 || !seq_len || dtype == UMB_SEQ_F32)
+    return UMB_EINVAL;
+  const dim3 grid((max_len + 15) / 16, B, G);
+  const size_t lds = 4 * (size_t)(2 * 32 * (D + 8) + 128) * sizeof(u16);
+#define PWA_MFMA_CASE(NS)                                                                                                  \
+  case NS:                                                                                                                 \
+    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)pwa_attend_mfma_kernel<P, NS>,                                 \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)        \
+      return UMB_EHIP;                                                                                                     \
+    hipLaunchKernelGGL((pwa_attend_mfma_kernel<P, NS>), grid, dim3(256), lds, st, (u16*)out, q, *kv, proj, ld, gate_col,   \
+                       (const u16*)pos_bias, seq_slot, seq_row0, seq_pos0, seq_len, H, G, window, pool, scale);            \
+    break;
+  if (dtype == UMB_SEQ_BF16) {
+    using P = BF16;
+    switch (D / 32) { PWA_MFMA_CASE(1) PWA_MFMA_CASE(2) PWA_MFMA_CASE(3) PWA_MFMA_CASE(4) PWA_MFMA_CASE(5) PWA_MFMA_CASE(6)
+                      PWA_MFMA_CASE(7) PWA_MFMA_CASE(8) default: return UMB_EINVAL; }
+  } else if (dtype == UMB_SEQ_F16) {
+    using P = F16;
+    switch (D / 32) { PWA_MFMA_CASE(1) PWA_MFMA_CASE(2) PWA_MFMA_CASE(3) PWA_MFMA_CASE(4) PWA_MFMA_CASE(5) PWA_MFMA_CASE(6)
+                      PWA_MFMA_CASE(7) PWA_MFMA_CASE(8) default: return UMB_EINVAL; }
+  } else {
+    return UMB_EINVAL;
+  }
+#undef PWA_MFMA_CASE
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }

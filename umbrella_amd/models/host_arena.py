@@ -5,9 +5,9 @@ and lets the allocator decide where the pages live.  On a two-socket host that d
 socket crosses the inter-socket fabric on its way to the GPU (round 4 measured 330 - 377 ms per step for the same 40
 streamed layers, by what the process had allocated before).  Here the slabs of a model come out of ONE arena:
 
-  * anonymous mmap, transparent huge pages requested (madvise), bound to the NUMA node of the GPU's PCIe root
-    (libnuma `numa_tonode_memory` = mbind MPOL_BIND; the node is read from sysfs), touched once, then pinned with ONE
-    hipHostRegister -- one registration instead of one per layer;
+  * ONE pinned allocation (hipHostMalloc) made while the allocating thread prefers the NUMA
+    node of the GPU's PCIe root (libnuma `numa_set_preferred`; the node is read from sysfs) and touched once there -- one
+    allocation instead of one per layer, and no registration of existing pages (hosts may refuse it);
   * `reserve()` lets a process claim the arena EARLY (bench.py does, before the headline's allocations fragment the
     host); a model that streams takes its slabs from the reserved arena when it fits, else from a fresh one;
   * every step that is not available (no libnuma, a single-node host, no sysfs entry) degrades to the next best thing
@@ -21,12 +21,6 @@ import weakref
 
 import torch
 
-_libc = C.CDLL(None, use_errno=True)
-_libc.mmap.restype = C.c_void_p
-_libc.mmap.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_long]
-_libc.munmap.argtypes = [C.c_void_p, C.c_size_t]
-_libc.madvise.argtypes = [C.c_void_p, C.c_size_t, C.c_int]
-PROT_RW, MAP_PRIVATE_ANON, MADV_HUGEPAGE = 0x1 | 0x2, 0x02 | 0x20, 14
 ALIGN = 2 << 20
 
 
@@ -48,6 +42,23 @@ def host_nodes() -> int:
         return 1
 
 
+HOST_MALLOC_NUMA_USER = 0x20000000      # hipHostMallocNumaUser: place the pages by the calling thread's NUMA policy
+_hip = None
+
+
+def _hip_runtime():
+    """the HIP runtime torch has already loaded, through ctypes (hipHostMalloc / hipHostFree only)"""
+    global _hip
+    if _hip is None:
+        _hip = C.CDLL("libamdhip64.so")
+        _hip.hipHostMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t, C.c_uint]
+        _hip.hipHostMalloc.restype = C.c_int
+        _hip.hipHostFree.argtypes = [C.c_void_p]
+        _hip.hipHostFree.restype = C.c_int
+        _hip.hipGetLastError.restype = C.c_int
+    return _hip
+
+
 class HostArena:
     def __init__(self, nbytes: int, device):
         self.size = (int(nbytes) + ALIGN - 1) // ALIGN * ALIGN
@@ -57,58 +68,63 @@ class HostArena:
             self.node = int(os.environ["UMB_HOST_ARENA_NODE"])
         self.nodes = host_nodes()
         self.notes = []
-        base = _libc.mmap(None, self.size, PROT_RW, MAP_PRIVATE_ANON, -1, 0)
-        if base in (None, C.c_void_p(-1).value):
-            raise MemoryError(f"mmap of {self.size} bytes failed (errno {C.get_errno()})")
-        self.base = base
-        if _libc.madvise(base, self.size, MADV_HUGEPAGE) != 0:
-            self.notes.append("no transparent huge pages")
-        self.bound = False
+        # The arena is ALLOCATED pinned (hipHostMalloc), never registered after the fact:
+        # registering existing pages (hipHostRegister) is refused on some hosts, and the error it leaves behind surfaces in
+        # whatever GPU call comes next.  Placement: the allocating thread prefers the GPU's NUMA node while the pages are
+        # first touched (libnuma numa_set_preferred; local allocation is restored right after).
+        numa, self.bound = None, False
         if self.node >= 0 and self.nodes > 1:
             try:
                 numa = C.CDLL("libnuma.so.1", use_errno=True)
-                numa.numa_tonode_memory.argtypes = [C.c_void_p, C.c_size_t, C.c_int]
                 if numa.numa_available() >= 0:
-                    # PREFERRED, not strict: numa_tonode_memory binds under libnuma's current bind policy, and under a strict
-                    # bind a node without `size` free bytes sends the first-touch memset below to the OOM killer instead of
-                    # to this constructor's caller.  Bind only when the node really has the room, and say what happened.
-                    numa.numa_set_bind_policy.argtypes = [C.c_int]
-                    numa.numa_set_bind_policy(0)
                     numa.numa_node_size64.argtypes = [C.c_int, C.POINTER(C.c_longlong)]
                     numa.numa_node_size64.restype = C.c_longlong
                     free = C.c_longlong(0)
                     total = numa.numa_node_size64(self.node, C.byref(free))
                     if total > 0 and free.value >= self.size + (1 << 30):
-                        C.set_errno(0)
-                        numa.numa_tonode_memory(base, self.size, self.node)      # (void in libnuma; failures surface in errno)
-                        if C.get_errno() == 0:
-                            self.bound = True
-                        else:
-                            self.notes.append(f"numa_tonode_memory errno {C.get_errno()}: first-touch placement")
+                        numa.numa_set_preferred.argtypes = [C.c_int]
+                        numa.numa_set_preferred(self.node)
+                        self.bound = True
                     else:
                         self.notes.append(f"node {self.node} has {free.value >> 20} MiB free of the {self.size >> 20} MiB wanted: "
                                           "first-touch placement")
+                else:
+                    numa = None
             except OSError:
+                numa = None
                 self.notes.append("libnuma missing: first-touch placement")
         elif self.nodes <= 1:
             self.notes.append("single NUMA node")
         else:
             self.notes.append("GPU NUMA node unknown")
-        C.memset(base, 0, self.size)                                     # first touch under the binding
-        rc = int(torch.cuda.cudart().cudaHostRegister(base, self.size, 0))
-        if rc != 0:
-            _libc.munmap(base, self.size)
-            raise RuntimeError(f"hipHostRegister failed ({rc})")
-        self.registered = True
+        # hipHostMalloc directly, not torch's caching pinned allocator: that one rounds a request up to a power of two
+        # (36 GB of slabs would pin 64) and keeps the block pinned after the model is gone
+        self.base = None
+        hip = _hip_runtime()
+        ptr = C.c_void_p()
+        try:
+            rc = hip.hipHostMalloc(C.byref(ptr), self.size + ALIGN, HOST_MALLOC_NUMA_USER if self.bound else 0)
+            if rc != 0 and self.bound:
+                hip.hipGetLastError()
+                rc = hip.hipHostMalloc(C.byref(ptr), self.size + ALIGN, 0)
+            if rc != 0 or not ptr.value:
+                hip.hipGetLastError()                                    # leave no sticky error behind for the next GPU call
+                raise MemoryError(f"hipHostMalloc of {self.size >> 20} MiB failed ({rc})")
+            self.base = ptr.value
+            C.memset(self.base, 0, self.size + ALIGN)                    # first touch under the preference
+        finally:
+            if numa is not None and self.bound:
+                numa.numa_set_localalloc()
+        self.skew = (-self.base) % ALIGN                                 # slabs start on 2 MiB boundaries
         self.off = 0
         self.live = 0
 
     def alloc(self, nbytes: int):
-        """a uint8 CPU tensor of nbytes inside the arena (2 MiB aligned), or None if it does not fit"""
+        """a pinned uint8 CPU tensor of nbytes inside the arena (2 MiB aligned), or None if it does not fit"""
         n = (int(nbytes) + ALIGN - 1) // ALIGN * ALIGN
-        if self.off + n > self.size:
+        if self.base is None or self.off + n > self.size:
             return None
-        buf = (C.c_uint8 * int(nbytes)).from_address(self.base + self.off)
+        buf = (C.c_uint8 * int(nbytes)).from_address(self.base + self.skew + self.off)
         t = torch.frombuffer(buf, dtype=torch.uint8)
         t._arena = self                                                  # the arena outlives its tensors
         self.off += n
@@ -124,15 +140,12 @@ class HostArena:
         self.off, self.live = 0, 0
 
     def describe(self) -> dict:
-        return {"arena": f"mmap {self.size >> 20} MiB, one hipHostRegister" + ("; " + "; ".join(self.notes) if self.notes else ""),
+        return {"arena": f"{self.size >> 20} MiB in one pinned allocation" + ("; " + "; ".join(self.notes) if self.notes else ""),
                 "numa_node": self.node, "host_numa_nodes": self.nodes, "bound_to_gpu_node": self.bound}
 
     def close(self):
-        if getattr(self, "registered", False):
-            torch.cuda.cudart().cudaHostUnregister(self.base)
-            self.registered = False
         if getattr(self, "base", None):
-            _libc.munmap(self.base, self.size)
+            _hip_runtime().hipHostFree(C.c_void_p(self.base))
             self.base = None
 
     def __del__(self):
