@@ -104,7 +104,7 @@ def test_linear_rows_do_not_depend_on_the_batch(lib):
 
 
 # ------------------------------------------------------------------ norms
-@pytest.mark.parametrize("groups,W", [(1, 40), (4, 64), (3, 201)])
+@pytest.mark.parametrize("groups,W", [(1, 40), (4, 64), (3, 201), (2, 1280), (1, 1100)])
 def test_group_norm_and_residual_seam(lib, groups, W):
     from oracle import seqmix as O
     from umbrella_amd import _lib
@@ -161,7 +161,8 @@ def _run_gla(X, w, H, D, E, tau, eps, state, slot, pos0, splits):
     return torch.cat(outs)
 
 
-@pytest.mark.parametrize("H,D,E,rank,tau", [(2, 16, 8, 4, 8.0), (3, 24, 20, 5, 1.0), (1, 130, 70, 16, 32.0), (2, 7, 3, 1, 2.5), (1, 256, 18, 3, 4.0)])
+@pytest.mark.parametrize("H,D,E,rank,tau", [(2, 16, 8, 4, 8.0), (3, 24, 20, 5, 1.0), (1, 130, 70, 16, 32.0), (2, 7, 3, 1, 2.5), (1, 256, 18, 3, 4.0),
+                                              (2, 64, 32, 8, 4.0), (1, 128, 16, 4, 16.0)])
 def test_gla_alone_prefill_and_token_by_token(lib, H, D, E, rank, tau):
     from oracle import seqmix as O
     width, n, eps = 40, 37, 1e-5
@@ -283,6 +284,23 @@ def test_attention_alone_every_position(lib, H, G, D, window, pool, rot_dims, pa
     assert (parts - whole).abs().max() < 1e-5
 
 
+def test_attention_many_rounds_of_keys(lib):
+    """a window and a pooled history that each span several 64-key rounds (and 32-key steps), in prompts and in decoding"""
+    H, G, D, window, pool, page, width, n, eps = 2, 1, 32, 100, 2, 16, 24, 300, 1e-5
+    w = _attn_weights(width, H, G, D, seed=77)
+    X = torch.randn(n, width, generator=torch.Generator().manual_seed(5))
+    kw = dict(H=H, G=G, D=D, window=window, pool=pool, rot_dims=16, base=1000.0, scale=0.1, eps=eps)
+    want = _attn_oracle(X, w, torch.float32, **kw)
+    whole, _ = _run_attn(X, w, dtype=torch.float32, page=page, splits=[n], **kw)
+    scale = float(want.abs().max())
+    assert (whole.cpu().double() - want).abs().max() < 2e-5 * scale
+    steps, _ = _run_attn(X, w, dtype=torch.float32, page=page, splits=[250] + [1] * 50, **kw)
+    assert (steps - whole).abs().max() < 2e-5 * scale
+    want16 = _attn_oracle(X, w, torch.bfloat16, **kw)
+    tiled, _ = _run_attn(X, w, dtype=torch.bfloat16, page=page, splits=[140, 160], tiled=True, **kw)
+    assert (tiled.cpu().double() - want16).abs().max() < 1.2e-2 * scale
+
+
 def _standout(n, width, H, G, D, loud):
     """weights and inputs under which every key is (almost) invisible except the tokens in `loud`, each of which has weight
     1/2 for every later query: constant projections, a strongly negative score bias, keys that point along the query for
@@ -320,7 +338,8 @@ def test_attention_window_and_pool_edges_with_standout_keys(lib, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("H,G,D,window,pool,rot_dims,page", [(4, 2, 32, 6, 3, 32, 4), (8, 2, 64, 9, 7, 16, 5), (3, 3, 32, 1, 1, 8, 3),
-                                                             (2, 1, 96, 20, 4, 0, 64)])
+                                                             (2, 1, 96, 20, 4, 0, 64), (2, 1, 128, 12, 5, 64, 8),
+                                                             (1, 1, 256, 7, 2, 256, 16)])
 def test_attention_on_the_matrix_pipe(lib, dtype, H, G, D, window, pool, rot_dims, page):
     """prompt stretches of >= 16 tokens through the MFMA kernel (every phase of window, block, page and 16-query tile),
     against the oracle and against the vector-pipe kernel: the two must agree to the rounding of their 16-bit outputs"""

@@ -114,6 +114,8 @@ class BatchEngine(BaseEngine):
         for rid, toks, w in entries:
             if rid not in cache.seqs:
                 m.open(rid)
+            if len(toks) == 0:                  # a request that brings nothing this step only keeps (or takes) its slot
+                continue
             parts.append((rid, toks))
             want.append(list(w))
         logits = m.forward_batch(parts, want=want) if parts else None
