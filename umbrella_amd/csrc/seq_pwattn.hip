@@ -111,7 +111,6 @@ __global__ __launch_bounds__(64) void pwa_pool_kernel(UmbPagedKV kv, const int* 
 // was cut.  Score phase: lane = key, 16-byte loads along the key's row against the queries held in LDS.  Value phase:
 // lane = value column, the round's weights broadcast one key at a time.
 constexpr int PWA_MAXC = 4;      // value columns per lane: D <= 256
-constexpr int PWA_KB = 8;        // keys whose value loads are in flight together
 
 template <typename P, int RH, int NC, int NW>
 __global__ __launch_bounds__(NW * 64) void pwa_attend_kernel(typename El<P>::type* __restrict__ out, const float* __restrict__ q,
@@ -121,6 +120,7 @@ __global__ __launch_bounds__(NW * 64) void pwa_attend_kernel(typename El<P>::typ
                                                          int G, int D, int window, int pool, float scale) {
   typedef typename El<P>::type E;
   extern __shared__ float lds[];
+  constexpr int PWA_KB = 8;   // keys whose value rows are in flight together (32 measured 3x slower at 16 waves: registers)
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int Dp = (D + 3) & ~3;
   float* q_s = lds;                                          // [RH][Dp] queries; later [NW][RH][Dp] partial outputs
