@@ -484,6 +484,39 @@ def test_model_long_decoding_and_first_tokens(lib):
     assert len(m.kv_cache.seqs["s"]["pages"]) == 25
 
 
+def test_decode_steps_replayed_as_graphs_equal_eager_launches(lib):
+    """decode steps of a batch size are captured once and replayed; between replays the cache manager hands out pages, a
+    request ends, a prompt of another request is prefilled eagerly: every replay must give what eager launches give"""
+    from seqmix_helpers import CONFIGS, build, tokens
+    cfgd = CONFIGS["mixed"]
+    V = cfgd["vocab"]
+    outs = []
+    for graph in (True, False):
+        from umbrella_amd.models import gitopel
+        cfg = gitopel.config_from_dict(cfgd)
+        sd = gitopel.synth_state(cfg, seed=13, rank=6)
+        m = gitopel.Gitopel("tiny", batch_size=4, max_length=128, max_tokens=512, device="cuda:0", dtype=torch.bfloat16,
+                            state_dict=sd, config=cfg, page_size=4, hip_graph=graph)
+        m.alloc()
+        got = []
+        for k in "abc":
+            m.open(k)
+        got.append(m.forward_batch([("a", tokens(9, V, 1)), ("b", tokens(3, V, 2)), ("c", tokens(17, V, 3))]).clone())
+        for i in range(10):                                    # three sequences: first step eager, second captured, then replays
+            got.append(m.forward_batch([(k, [(7 * i + j) % V]) for j, k in enumerate("abc")]).clone())
+        m.close("b")
+        m.open("d")
+        got.append(m.forward_batch([("d", tokens(6, V, 4))]).clone())            # eager work between replays
+        for i in range(6):                                     # the same batch size again, another sequence in the slot
+            got.append(m.forward_batch([(k, [(5 * i + j) % V]) for j, k in enumerate("adc")]).clone())
+        for i in range(3):                                     # another batch size: its own graph
+            got.append(m.forward_batch([(k, [(3 * i + j) % V]) for j, k in enumerate("ad")], want=[[0], []]).clone())
+        assert (len(m._graphs) >= 2 and all(e["graph"] is not None for e in m._graphs.values())) == graph
+        outs.append(got)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
 def test_cache_runs_out_loudly_and_recovers(lib):
     from seqmix_helpers import CONFIGS, build, tokens
     m, _ = build(CONFIGS["mixed"], torch.bfloat16, page=4, batch=2, max_tokens=16, max_length=64)

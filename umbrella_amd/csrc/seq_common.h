@@ -38,3 +38,16 @@ __device__ __forceinline__ long pkv_blk(const UmbPagedKV& kv, int slot, int b, i
   const int npb = (kv.page + pool - 1) / pool;
   return (((long)pg * G + g) * npb + (e % kv.page) / pool) * D;
 }
+
+// Dynamic LDS above the default limit needs the function attribute.  It is set once per kernel and size (a function-local
+// static per kernel instantiation), i.e. by the first eager launch: a step that is being captured into a hipGraph has run
+// eagerly before and makes no such call.
+template <auto Kernel> static inline int ensure_dynamic_lds(size_t bytes) {
+  static size_t granted = 48 * 1024;
+  if (bytes > granted) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+      return UMB_EHIP;
+    granted = bytes;
+  }
+  return UMB_OK;
+}

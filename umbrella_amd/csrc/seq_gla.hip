@@ -222,9 +222,7 @@ extern "C" int umb_gla_scan(float* o, float* state, const float* proj, int ld, c
   const bool v4 = D % 4 == 0 && Dv % 4 == 0 && ld % 4 == 0;
 #define GLA_SCAN_LAUNCH(NR, V4)                                                                                           \
   do {                                                                                                                    \
-    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)gla_scan_kernel<NR, V4>,                                      \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)       \
-      return UMB_EHIP;                                                                                                    \
+    if (ensure_dynamic_lds<gla_scan_kernel<NR, V4>>(lds) != UMB_OK) return UMB_EHIP;                                      \
     hipLaunchKernelGGL((gla_scan_kernel<NR, V4>), grid, dim3(256), lds, st, o, state, proj, ld, alpha, seq_slot, seq_row0, \
                        seq_pos0, seq_len, H, D, Dv, qscale);                                                              \
   } while (0)

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
     for (int nt = 0; nt < NT; ++nt) { acc[nt][tt] = f32x4{0.f, 0.f, 0.f, 0.f}; acc2[nt][tt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
   }
 
-  constexpr int UN = (NT * TT == 1) ? 8 : 2;        // 32-k steps in flight per wave (a single-tile launch is latency-bound:
+  constexpr int UN = (NT * TT == 1) ? (DUAL ? 8 : 16) : 2;        // 32-k steps in flight per wave (a single-tile launch is latency-bound:
                                                     // K = 2048 is two round trips per wave instead of four)
   for (int k0 = wave * 32; k0 < K; k0 += 128 * UN) {
     Frag8<P> a[UN][NT], a2[UN][NT], b[UN][TT];

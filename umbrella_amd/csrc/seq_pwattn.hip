@@ -501,11 +501,15 @@ extern "C" int umb_pwa_attend(void* out, const float* q, const UmbPagedKV* kv, c
   const dim3 grid(T, H / rh);
   // few workgroups (decoding): sixteen waves share a query's keys, so a step's latency is one or two rounds; many (prompts):
   // four, the chip is full anyway.  The choice changes the order in which a query's partial sums are added, nothing else.
-  const int nw = (long)T * (H / rh) < 1024 ? 16 : 4;
+  int nw = (long)T * (H / rh) < 1024 ? 16 : 4;
+  if (nw == 16 && ((size_t)16 * rh * Dp + 16 * (rh * 64 + 128)) * sizeof(float) > 96 * 1024) nw = 4;     // LDS of one CU
   const size_t lds = ((size_t)nw * rh * Dp + nw * (rh * 64 + 128)) * sizeof(float);
 #define PWA_LAUNCH(RH, NC, NW)                                                                                            \
-  hipLaunchKernelGGL((pwa_attend_kernel<P, RH, NC, NW>), grid, dim3(NW * 64), lds, st, (E*)out, q, *kv, proj, ld, gate_col, \
-                     (const E*)pos_bias, pos, slot, T, H, G, D, window, pool, scale)
+  do {                                                                                                                    \
+    if (ensure_dynamic_lds<pwa_attend_kernel<P, RH, NC, NW>>(lds) != UMB_OK) return UMB_EHIP;                             \
+    hipLaunchKernelGGL((pwa_attend_kernel<P, RH, NC, NW>), grid, dim3(NW * 64), lds, st, (E*)out, q, *kv, proj, ld,       \
+                       gate_col, (const E*)pos_bias, pos, slot, T, H, G, D, window, pool, scale);                         \
+  } while (0)
 #define PWA_NC(RH, NW)                                                                                                    \
   if (D <= 64) PWA_LAUNCH(RH, 1, NW); else if (D <= 128) PWA_LAUNCH(RH, 2, NW); else PWA_LAUNCH(RH, 4, NW)
 #define PWA_CASE(RH)                                                                                                       \
@@ -534,9 +538,7 @@ extern "C" int umb_pwa_attend_tiled(void* out, const float* q, const UmbPagedKV*
   const size_t lds = 4 * (size_t)(2 * 32 * (D + 8) + 128) * sizeof(u16);
 #define PWA_MFMA_CASE(NS)                                                                                                  \
   case NS:                                                                                                                 \
-    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)pwa_attend_mfma_kernel<P, NS>,                                 \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)        \
-      return UMB_EHIP;                                                                                                     \
+    if (ensure_dynamic_lds<pwa_attend_mfma_kernel<P, NS>>(lds) != UMB_OK) return UMB_EHIP;                                 \
     hipLaunchKernelGGL((pwa_attend_mfma_kernel<P, NS>), grid, dim3(256), lds, st, (u16*)out, q, *kv, proj, ld, gate_col,   \
                        (const u16*)pos_bias, seq_slot, seq_row0, seq_pos0, seq_len, H, G, window, pool, scale);            \
     break;
