@@ -26,7 +26,9 @@ extern "C" {
 typedef struct ihipStream_t* umb_stream_t;   /* == hipStream_t */
 
 enum { UMB_SEQ_F16 = 0, UMB_SEQ_BF16 = 1, UMB_SEQ_F32 = 2 };
-enum { UMB_MIX_POOLED_WINDOW = 0, UMB_MIX_GLA = 1 };
+enum { UMB_MIX_POOLED_WINDOW = 0, UMB_MIX_GLA = 1, UMB_MIX_LATENT = 2 };
+/* feed-forward kinds: gated SiLU (W_down (silu(W_gate h) * W_up h)), PolyNorm (W_down polynorm(W_up h)), routed experts */
+enum { UMB_FF_GATED = 0, UMB_FF_POLYNORM = 1, UMB_FF_MOE = 2 };
 
 /* W [N][K] row-major (as stored: out x in), optional bias [N]; applied as W x + b */
 typedef struct UmbSeqLinear { const void* w; const void* bias; int32_t N, K; } UmbSeqLinear;
@@ -39,6 +41,18 @@ typedef struct UmbSeqLinear { const void* w; const void* bias; int32_t N, K; } U
 int umb_seq_linear(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, int dtype,
                    umb_stream_t stream);
 
+/* The same product for `batch` independent problems (blockIdx.z): problem b reads x + b sx (rows ldx apart), weights
+ * w + b sw ([N][K]) and writes out + b so (rows ldo apart); strides in elements; no bias.  epi 0 / 1 as above;
+ * epi 3: out in `dtype` = acc * sigmoid(gate[t ldg + b sg + n]) (gate fp32).  The K order of an output is that of
+ * umb_seq_linear. */
+int umb_seq_linear_batched(void* out, const void* x, const void* w, int T, int N, int K, int ldx, int ldo, int batch, long sx,
+                           long sw, long so, int epi, const float* gate, int ldg, int sg, int dtype, umb_stream_t stream);
+/* Grouped product over row ranges read from device memory: tile i (blockIdx.y, i < max_tiles) is {group, first row, rows}
+ * (3 int32, rows <= 64, rows == 0: nothing); its rows of x [*][K] meet w + group * gs ([N][K], or the stacked [2N'][K] of
+ * epi 2) and land in the same rows of out.  No bias. */
+int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, long gs, int N, int K,
+                           int epi, int dtype, umb_stream_t stream);
+
 /* RMS norm in `groups` equal consecutive parts of a row: part / sqrt(mean(part^2) + eps), whole row times w.
  * x fp32 [*][W]; rows: optional gather (row i of out comes from row rows[i] of x); out_f32 and/or out_dt may be given. */
 int umb_seq_group_norm(float* out_f32, void* out_dt, const float* x, const int* rows, const void* w, int T, int W, int groups,
@@ -49,6 +63,40 @@ int umb_seq_embed_norm(float* x, void* h, const void* embed, const int* tokens, 
 /* x <- x + group_norm(y) * w_post ; if w_next: h <- group_norm(x) * w_next in `dtype`   (y fp32 [T][W]) */
 int umb_seq_resid_norm(float* x, void* h, const float* y, const void* w_post, const void* w_next, int T, int W, int groups,
                        float eps, int dtype, umb_stream_t stream);
+
+/* x[t] <- embed[tokens[t]] * scale (fp32) */
+int umb_seq_embed(float* x, const void* embed, const int* tokens, float scale, int T, int W, int V, int dtype,
+                  umb_stream_t stream);
+
+/* ---- causal convolution over time in front of a sublayer ("canon"): h[t] = x[t] + sum_j w[c][j] x(p - taps + 1 + j), the
+ * sum over the `taps` positions up to and including the token's own position p; positions before the sequence's start are
+ * zero, positions of earlier steps come from the sequence's state.  x fp32 [T][W]; w [W][taps]; h in `dtype`.
+ * state fp32 [slots][taps - 1][W]: the input at position p lives in row p % (taps - 1).  The convolution reads the state;
+ * `umb_canon_update`, launched after it, stores the step's last inputs. taps == 1 needs no state. */
+int umb_canon_conv(void* h, const float* x, const void* w, const float* state, const int* pos, const int* slot, int T, int W,
+                   int taps, int dtype, umb_stream_t stream);
+int umb_canon_update(float* state, const float* x, const int* seq_slot, const int* seq_row0, const int* seq_pos0,
+                     const int* seq_len, int B, int W, int taps, umb_stream_t stream);
+/* one launch for steps of one token per sequence: convolution and state update by the same thread */
+int umb_canon_step(void* h, const float* x, const void* w, float* state, const int* pos, const int* slot, int T, int W,
+                   int taps, int dtype, umb_stream_t stream);
+
+/* ---- PolyNorm activation: out[t] = a N(z) + b N(z^2) + c N(z^3) + e with powers element by element and
+ * N(v) = v / sqrt(mean(v^2) + eps) over the row; coef = {a, b, c, e} in `dtype`; z fp32 [T][F], out in `dtype`. */
+int umb_polynorm(void* out, const float* z, const void* coef, int T, int F, float eps, int dtype, umb_stream_t stream);
+
+/* ---- routed experts.  logits fp32 [T][E]; scores = sigmoid(logits); each token keeps its `top` largest (ties: the lower
+ * index), weight = the score itself.  sel [T][top] expert ids, wt [T][top] fp32. */
+int umb_moe_route(int* sel, float* wt, const float* logits, int T, int E, int top, umb_stream_t stream);
+/* orders the T*top (token, choice) pairs by expert: pos_of [T*top] = row of the pair in the expert-ordered list,
+ * tiles [max_tiles][3] = {expert, first row, rows} covering every expert's rows in pieces of at most 64
+ * (max_tiles >= ceil(T top / 64) + E; unused entries get rows = 0). */
+int umb_moe_plan(int* pos_of, int* tiles, const int* sel, int T, int E, int top, int max_tiles, umb_stream_t stream);
+/* xs[pos_of[t top + k]] = wt[t][k] * h[t]  (the weight multiplies the expert's INPUT); h, xs in `dtype` */
+int umb_moe_scatter(void* xs, const void* h, const float* wt, const int* pos_of, int T, int W, int top, int dtype,
+                    umb_stream_t stream);
+/* y[t] = (add ? y[t] : 0) + sum_k ye[pos_of[t top + k]]  (k ascending) */
+int umb_moe_combine(float* y, const float* ye, const int* pos_of, int T, int W, int top, int add, umb_stream_t stream);
 
 /* ---- gated linear attention.  proj fp32 [T][ld]: columns [q (H D) | k (H D) | v (H Dv) | g (H Dv) | a (rank)].
  * decay: alpha[t][H D] = sigmoid(W_a2 a + b)^(1/tau), fp32 */
@@ -92,6 +140,32 @@ int umb_pwa_attend_tiled(void* out, const float* q, const UmbPagedKV* kv, const 
                          int B, int max_len, int H, int G, int D, int window, int pool, float scale, int dtype,
                          umb_stream_t stream);
 
+/* ---- latent attention: queries and keys/values go through low-rank latents; the cache holds, per token, the normed
+ * key/value latent c [kv_rank] and one rotated key part [rot_dim] shared by all heads (one row of kv_rank + rot_dim in
+ * `dtype`; pages as above, UmbPagedKV.k only, one "head").  Scores and values are taken against c itself:
+ *   score(i, j, h) = (q_lat[i][h] . c[j] + q_rot[i][h] . k_rot[j]) * scale,   q_lat = W_uk[h]^T q_nope
+ *   out[i][h]      = W_uv[h] (sum_j p[i][j][h] c[j]),
+ * which equals attention over per-head keys W_uk[h] c and values W_uv[h] c without ever forming them.
+ * lat_prep: proj fp32 [T][ld] = [dq (q_rank) | dkv (kv_rank + rot_dim) | ...]; cq = rms_norm(dq) * w_q in `dtype`;
+ * cache row = [rms_norm(dkv[:kv_rank]) * w_kv | rope(dkv[kv_rank:])]. */
+int umb_lat_prep(void* cq, const UmbPagedKV* kv, const float* proj, int ld, const void* w_q, const void* w_kv, const int* pos,
+                 const int* slot, const float* freq, int T, int q_rank, int kv_rank, int rot_dim, int rot_dims, float eps,
+                 int dtype, umb_stream_t stream);
+/* q fp32 [T][H (D + R)] head by head [unrotated D | rotated R] -> qn [T][H D] in `dtype` (unrotated parts) and
+ * qa[t][h][kv_rank ..] = rope(rotated part) fp32 (qa fp32 [T][H][kv_rank + R]; the first kv_rank come from the
+ * batched product with W_uk^T) */
+int umb_lat_qsplit(void* qn, float* qa, const float* q, const int* pos, const float* freq, int T, int H, int D, int R,
+                   int kv_rank, int rot_dims, int dtype, umb_stream_t stream);
+/* softmax attention of qa over the cached rows of the window (0 <= i - j < window) with a sink per head in the
+ * denominator (exp(sink[h]): no key, no value, not scaled; sink may be null); out [T][H][kv_rank] in `dtype`. */
+int umb_lat_attend(void* out, const float* qa, const UmbPagedKV* kv, const void* sink, const int* pos, const int* slot, int T,
+                   int H, int kv_rank, int rot_dim, int window, float scale, int dtype, umb_stream_t stream);
+/* the same for steps that bring stretches of a sequence, on the matrix pipe: workgroups own 16 consecutive positions of
+ * one sequence.  umb_lat_attend_tiled_ok says (1 / 0) whether the kernel covers a shape and dtype; it has no stream. */
+int umb_lat_attend_tiled(void* out, const float* qa, const UmbPagedKV* kv, const void* sink, const int* seq_slot,
+                         const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int max_len, int H, int kv_rank,
+                         int rot_dim, int window, float scale, int dtype, umb_stream_t stream);
+
 /* ------------------------------------------------------------------ the model */
 typedef struct UmbSeqLayer {
   int32_t kind, has_mlp;
@@ -105,15 +179,33 @@ typedef struct UmbSeqLayer {
   UmbSeqLinear gu, down;  /* feed-forward: stacked [gate; up], down */
   const void* pos_bias;   /* attention: [heads] */
   const void* head_norm;  /* GLA: [vdim] */
+  /* x <- x + norm1b(mixer(norm1(x))), x <- x + norm2b(ff(norm2(x))); norm1 / norm2 null: the sublayer reads the
+   * residual stream itself (through the convolution below) */
   const void *norm1, *norm1b, *norm2, *norm2b;
   const float* rot_freq;  /* [rot_dims / 2] fp32 */
   UmbPagedKV kv;          /* attention layers */
   float* state;           /* GLA layers: [slots][heads][dim][vdim] fp32 */
+  /* latent attention (proj = [dq | dkv | gate]) */
+  int32_t q_rank, kv_rank, rot_dim, ff_kind;
+  /* routed experts */
+  int32_t experts, top, expert_ff, shared_ff;
+  UmbSeqLinear uq;        /* [heads (dim + rot_dim)][q_rank] */
+  const void* uk_t;       /* [heads][kv_rank][dim]: W_uk of every head, transposed */
+  const void* uv;         /* [heads vdim][kv_rank] */
+  const void *dq_norm, *dkv_norm, *sink;
+  /* convolution in front of the sublayers: weights [W][taps], state [slots][taps - 1][W] fp32 (null: none) */
+  const void *canon1, *canon2;
+  float *canon_state1, *canon_state2;
+  const void* act;        /* PolyNorm: {a, b, c, e} */
+  UmbSeqLinear router;    /* [experts][W] */
+  const void* e_gu;       /* [experts][2 expert_ff][W]: every expert's stacked [gate; up] */
+  const void* e_down;     /* [experts][W][expert_ff] */
+  UmbSeqLinear s_gu, s_down;   /* shared expert (s_gu.w null: none) */
 } UmbSeqLayer;
 
 typedef struct UmbSeqModel {
-  int32_t dtype, L, W, V, groups, pad_;
-  float eps, pad2_;
+  int32_t dtype, L, W, V, groups, canon_taps;
+  float eps, embed_scale;    /* embed_scale: the embedding row is multiplied by it (1: as stored) */
   const void* embed; const void* final_norm; UmbSeqLinear head;
   const UmbSeqLayer* layers;
 } UmbSeqModel;
@@ -130,6 +222,15 @@ typedef struct UmbSeqWork {
   float* y;        /* sublayer output [Tmax][W] fp32 */
   float* logits;   /* [Rmax][V] fp32 */
   int32_t Tmax, Rmax;
+  /* routed experts (null when no layer has any): pairs = Tmax * max top */
+  int32_t* moe_sel;   /* [pairs] */
+  float* moe_wt;      /* [pairs] */
+  int32_t* moe_pos;   /* [pairs] */
+  int32_t* moe_tiles; /* [moe_max_tiles][3] */
+  void* moe_xs;       /* [pairs][W] dtype */
+  void* moe_act;      /* [pairs][max expert_ff] dtype */
+  float* moe_y;       /* [pairs][W] fp32 */
+  int64_t moe_max_tiles;
 } UmbSeqWork;
 
 typedef struct UmbSeqStep {
@@ -139,6 +240,8 @@ typedef struct UmbSeqStep {
   const int32_t* logit_rows;                                /* [R] rows whose logits are wanted */
   float* trace;                                             /* optional [L][T][W]: the residual stream after every layer */
 } UmbSeqStep;
+
+int umb_lat_attend_tiled_ok(int H, int kv_rank, int rot_dim, int dtype);
 
 int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const UmbSeqStep* s, umb_stream_t stream);
 

@@ -126,7 +126,7 @@ class UmbOffload(C.Structure):
                 ("prefetched", C.POINTER(C.c_int32)), ("n_slabs", C.c_int32), ("pad_", C.c_int32)]
 
 
-_P, _I, _F = C.c_void_p, C.c_int, C.c_float
+_P, _I, _F, _L = C.c_void_p, C.c_int, C.c_float, C.c_long
 # name -> argtypes (all return int unless listed in _VOID / _STR)
 SIGNATURES = {
     "umb_repack_dense": [_P, _P, _I, _I, _I, _I, _I, _I, _P],
@@ -219,19 +219,27 @@ class UmbSeqLayer(C.Structure):
                 ("proj", UmbSeqLinear), ("a2", UmbSeqLinear), ("out", UmbSeqLinear), ("gu", UmbSeqLinear),
                 ("down", UmbSeqLinear), ("pos_bias", C.c_void_p), ("head_norm", C.c_void_p), ("norm1", C.c_void_p),
                 ("norm1b", C.c_void_p), ("norm2", C.c_void_p), ("norm2b", C.c_void_p), ("rot_freq", C.c_void_p),
-                ("kv", UmbPagedKV), ("state", C.c_void_p)]
+                ("kv", UmbPagedKV), ("state", C.c_void_p),
+                ("q_rank", C.c_int32), ("kv_rank", C.c_int32), ("rot_dim", C.c_int32), ("ff_kind", C.c_int32),
+                ("experts", C.c_int32), ("top", C.c_int32), ("expert_ff", C.c_int32), ("shared_ff", C.c_int32),
+                ("uq", UmbSeqLinear), ("uk_t", C.c_void_p), ("uv", C.c_void_p), ("dq_norm", C.c_void_p),
+                ("dkv_norm", C.c_void_p), ("sink", C.c_void_p), ("canon1", C.c_void_p), ("canon2", C.c_void_p),
+                ("canon_state1", C.c_void_p), ("canon_state2", C.c_void_p), ("act", C.c_void_p), ("router", UmbSeqLinear),
+                ("e_gu", C.c_void_p), ("e_down", C.c_void_p), ("s_gu", UmbSeqLinear), ("s_down", UmbSeqLinear)]
 
 
 class UmbSeqModel(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("L", C.c_int32), ("W", C.c_int32), ("V", C.c_int32), ("groups", C.c_int32),
-                ("pad_", C.c_int32), ("eps", C.c_float), ("pad2_", C.c_float), ("embed", C.c_void_p),
+                ("canon_taps", C.c_int32), ("eps", C.c_float), ("embed_scale", C.c_float), ("embed", C.c_void_p),
                 ("final_norm", C.c_void_p), ("head", UmbSeqLinear), ("layers", C.POINTER(UmbSeqLayer))]
 
 
 class UmbSeqWork(C.Structure):
     _fields_ = [("x", C.c_void_p), ("h", C.c_void_p), ("proj", C.c_void_p), ("aux", C.c_void_p), ("o", C.c_void_p),
                 ("mix", C.c_void_p), ("act", C.c_void_p), ("y", C.c_void_p), ("logits", C.c_void_p),
-                ("Tmax", C.c_int32), ("Rmax", C.c_int32)]
+                ("Tmax", C.c_int32), ("Rmax", C.c_int32), ("moe_sel", C.c_void_p), ("moe_wt", C.c_void_p),
+                ("moe_pos", C.c_void_p), ("moe_tiles", C.c_void_p), ("moe_xs", C.c_void_p), ("moe_act", C.c_void_p),
+                ("moe_y", C.c_void_p), ("moe_max_tiles", C.c_int64)]
 
 
 class UmbSeqStep(C.Structure):
@@ -244,6 +252,22 @@ class UmbSeqStep(C.Structure):
 _PKV = C.POINTER(UmbPagedKV)
 SEQ_SIGNATURES = {
     "umb_seq_linear": [_P, _P, _P, _P, _I, _I, _I, _I, _I],
+    "umb_seq_linear_batched": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _L, _I, _P, _I, _I, _I],
+    "umb_seq_linear_grouped": [_P, _P, _P, _P, _I, _L, _I, _I, _I, _I],
+    "umb_seq_embed": [_P, _P, _P, _F, _I, _I, _I, _I],
+    "umb_canon_conv": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I],
+    "umb_canon_update": [_P, _P, _P, _P, _P, _P, _I, _I, _I],
+    "umb_canon_step": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I],
+    "umb_polynorm": [_P, _P, _P, _I, _I, _F, _I],
+    "umb_moe_route": [_P, _P, _P, _I, _I, _I],
+    "umb_moe_plan": [_P, _P, _P, _I, _I, _I, _I],
+    "umb_moe_scatter": [_P, _P, _P, _P, _I, _I, _I, _I],
+    "umb_moe_combine": [_P, _P, _P, _I, _I, _I, _I],
+    "umb_lat_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I],
+    "umb_lat_qsplit": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
+    "umb_lat_attend": [_P, _P, _PKV, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I],
+    "umb_lat_attend_tiled": [_P, _P, _PKV, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I],
+    "umb_lat_attend_tiled_ok": [_I, _I, _I, _I],
     "umb_seq_group_norm": [_P, _P, _P, _P, _P, _I, _I, _I, _F, _I],
     "umb_seq_embed_norm": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I],
     "umb_seq_resid_norm": [_P, _P, _P, _P, _P, _I, _I, _I, _F, _I],
@@ -259,6 +283,7 @@ SEQ_SIGNATURES = {
     "umb_sample_rows": [_P, _P, _I, _I, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P],
     "umb_seq_version": [],
 }
+_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok"}          # predicates: no stream argument, the value is the answer
 _seq_lib = None
 
 
@@ -276,6 +301,8 @@ def load_seq() -> C.CDLL:
         fn = getattr(lib, name)
         if name == "umb_seq_version":
             fn.argtypes, fn.restype = [], C.c_char_p
+        elif name in _SEQ_NO_STREAM:
+            fn.argtypes, fn.restype = list(args), C.c_int
         else:
             fn.argtypes, fn.restype = list(args) + [_P], C.c_int
     _seq_lib = lib

@@ -145,14 +145,19 @@ class PagedSeqCache:
     * its tokens live in PAGES of ``page`` positions handed out on demand by ``extend`` and returned by ``close``; the same
       page numbers index every windowed-attention layer's K / V ``[pages, G, page, D]`` (storage dtype) and its pooled K / V
       ``[pages, G, ceil(page / pool), D]`` (fp32; a block lives in the page of its last position);
-    * gated-linear-attention layers keep one fp32 state ``[slots, H, D, Dv]`` each; nothing is cleared when a slot or a page
-      is handed out again: a sequence that starts at position 0 ignores what its slot holds, and no kernel reads a cache
-      position its own sequence has not written.
+    * latent-attention layers keep ONE row per token, ``[pages, page, kv_rank + rot_dim]`` (storage dtype): the normed
+      key/value latent and the rotated key part that all heads share;
+    * gated-linear-attention layers keep one fp32 state ``[slots, H, D, Dv]`` each;
+    * a convolution in front of a sublayer keeps its last ``taps - 1`` inputs, fp32 ``[slots, taps - 1, W]`` per sublayer
+      (the input at position p in row p % (taps - 1));
+    * nothing is cleared when a slot or a page is handed out again: a sequence that starts at position 0 ignores what its
+      slot holds, and no kernel reads a cache position its own sequence has not written.
 
     Free pages and slots are LIFO stacks, so whatever was given back last is used first.
     """
 
-    def __init__(self, kv_layers, state_layers, max_tokens: int, max_seqs: int, device, dtype, page: int = 64):
+    def __init__(self, kv_layers, state_layers, max_tokens: int, max_seqs: int, device, dtype, page: int = 64,
+                 latent_layers=(), conv_states: int = 0, conv_taps: int = 0, width: int = 0):
         assert page >= 1 and max_tokens >= 1 and max_seqs >= 1
         self.page, self.max_seqs, self.device, self.dtype = int(page), int(max_seqs), device, dtype
         # every sequence may leave one page partly filled
@@ -169,6 +174,9 @@ class PagedSeqCache:
                 vp=torch.zeros(self.n_pages, G, npb, D, dtype=torch.float32, device=device), G=G, D=D, pool=pool))
         for (H, D, Dv) in state_layers:
             self.state.append(torch.zeros(max_seqs, H, D, Dv, dtype=torch.float32, device=device))
+        self.latent = [torch.zeros(self.n_pages, page, Dk, dtype=dtype, device=device) for Dk in latent_layers]
+        self.conv = [torch.zeros(max_seqs, max(conv_taps - 1, 1), width, dtype=torch.float32, device=device)
+                     for _ in range(conv_states)] if conv_taps > 0 else []
         self.clear()
 
     def clear(self):
@@ -238,6 +246,19 @@ class PagedSeqCache:
         pg = torch.tensor(s["pages"], dtype=torch.long)[e // self.page].to(self.device)
         idx = ((e % self.page) // c["pool"]).to(self.device)
         return c["kp"][pg, :, idx], c["vp"][pg, :, idx]
+
+    def latent_rows(self, layer: int, seq_id, positions):
+        """cached latent rows of a sequence's positions -> [len(positions), kv_rank + rot_dim]"""
+        s = self.seqs[seq_id]
+        pos = torch.as_tensor(positions, dtype=torch.long)
+        pg = torch.tensor(s["pages"], dtype=torch.long)[pos // self.page].to(self.device)
+        return self.latent[layer][pg, (pos % self.page).to(self.device)]
+
+    def latent_struct(self, layer: int) -> "_lib.UmbPagedKV":
+        kv = _lib.UmbPagedKV()
+        kv.k, kv.v, kv.kp, kv.vp = self.latent[layer].data_ptr(), None, None, None
+        kv.pages, kv.max_pages, kv.page, kv.n_pages = self.pages_dev.data_ptr(), self.max_pages, self.page, self.n_pages
+        return kv
 
     def struct(self, layer: int) -> "_lib.UmbPagedKV":
         c = self.kv[layer]

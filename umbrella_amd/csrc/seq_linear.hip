@@ -56,7 +56,19 @@ template <> __device__ __forceinline__ f32x4 mma8<F32>(const Frag8<F32>& a, cons
   return c;
 }
 
-enum { EPI_F32 = 0, EPI_DT = 1, EPI_SILU_MUL = 2 };
+enum { EPI_F32 = 0, EPI_DT = 1, EPI_SILU_MUL = 2, EPI_GATE = 3 };
+
+// Where a launch departs from the dense [T][K] x [N][K] problem: row strides of x and out, a batch of independent problems
+// along blockIdx.z (element strides sx / sw / so), or token tiles read from device memory (grouped: tile blockIdx.y is
+// {group, first row, rows}; its weights start at w + group * gs).  EPI_GATE multiplies by sigmoid(gate[t ldg + z sg + n]).
+struct LinExt {
+  int ldx, ldo;
+  long sx, sw, so, gs;
+  const int* tiles;
+  const float* gate;
+  int ldg, sg;
+};
+static inline LinExt lin_dense(int N, int K) { return LinExt{K, N, 0, 0, 0, 0, nullptr, nullptr, 0, 0}; }
 
 // NT output tiles x TT token tiles of 16 per workgroup (each wave holds all NT x TT accumulator tiles of its K share: one weight
 // fragment meets TT token fragments and one token fragment NT weight fragments, so a launch of many tokens moves
@@ -66,13 +78,28 @@ template <typename P, int NT, int TT, bool VEC, bool DUAL>
 __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_, const typename El<P>::type* __restrict__ x,
                                                          const typename El<P>::type* __restrict__ w,
                                                          const typename El<P>::type* __restrict__ bias, int T, int N, int K,
-                                                         int epi) {
+                                                         int epi, LinExt ext) {
   typedef typename El<P>::type E;
   static_assert(!DUAL || NT <= 2, "gate and up partials of NT x TT tiles must fit the LDS");
   __shared__ float red[DUAL ? 2 : 1][4][NT * TT][256];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int j = lane & 15, g = lane >> 4;
-  const int t0 = blockIdx.y * (TT * 16);
+  int t0 = blockIdx.y * (TT * 16);
+  const int ldx = ext.ldx, ldo = ext.ldo;
+  long obase = (long)blockIdx.z * ext.so;
+  const float* gate = ext.gate ? ext.gate + (long)blockIdx.z * ext.sg : nullptr;
+  x += (long)blockIdx.z * ext.sx;
+  w += (long)blockIdx.z * ext.sw;
+  if (ext.tiles) {                         // grouped: this workgroup's rows and weights come from the tile list
+    const int* td = ext.tiles + 3 * blockIdx.y;
+    const int rows = td[2];
+    if (rows <= 0) return;
+    w += (long)td[0] * ext.gs;
+    x += (long)td[1] * ldx;
+    obase += (long)td[1] * ldo;
+    T = rows;
+    t0 = 0;
+  }
   const E* wrow[NT];
   bool n_ok[NT];
 #pragma unroll
@@ -88,7 +115,7 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
   for (int tt = 0; tt < TT; ++tt) {
     const int t = t0 + tt * 16 + j;
     t_ok[tt] = t < T;
-    xrow[tt] = x + (long)(t_ok[tt] ? t : 0) * K;
+    xrow[tt] = x + (long)(t_ok[tt] ? t : 0) * ldx;
   }
   f32x4 acc[NT][TT], acc2[NT][TT];
 #pragma unroll
@@ -154,11 +181,13 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
 #pragma unroll
         for (int ww = 1; ww < 4; ++ww) u += red[1][ww][nt * TT + tt][threadIdx.x];
         u += bv2;
-        stf<P>(reinterpret_cast<E*>(out_) + (long)t * N + n, siluf_(s) * u);
+        stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, siluf_(s) * u);
       } else if (epi == EPI_DT) {
-        stf<P>(reinterpret_cast<E*>(out_) + (long)t * N + n, s);
+        stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, s);
+      } else if (epi == EPI_GATE) {
+        stf<P>(reinterpret_cast<E*>(out_) + obase + (long)t * ldo + n, s / (1.f + expf(-gate[(long)t * ext.ldg + n])));
       } else {
-        reinterpret_cast<float*>(out_)[(long)t * N + n] = s;
+        reinterpret_cast<float*>(out_)[obase + (long)t * ldo + n] = s;
       }
     }
   }
@@ -285,32 +314,36 @@ static int launch_wide(void* out, const void* x, const void* w, const void* bias
   }
 }
 
+// gy > 0: the number of token tiles is given (grouped launches); gz: independent problems
 template <typename P, int NT, int TT, bool VEC>
-static int launch_tt(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st) {
+static int launch_tt(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st,
+                     const LinExt& ext, int gy = 0, int gz = 1) {
   typedef typename El<P>::type E;
   constexpr int NTD = NT > 2 ? 2 : NT;             // gate/up: two tile pairs at most
-  const dim3 grid((N + NT * 16 - 1) / (NT * 16), (T + TT * 16 - 1) / (TT * 16));
+  const dim3 grid((N + NT * 16 - 1) / (NT * 16), gy > 0 ? gy : (T + TT * 16 - 1) / (TT * 16), gz);
   if (epi == EPI_SILU_MUL)
-    hipLaunchKernelGGL((seq_linear_kernel<P, NTD, TT, VEC, true>), dim3((N + NTD * 16 - 1) / (NTD * 16), grid.y), dim3(256), 0, st,
-                       out, (const E*)x, (const E*)w, (const E*)bias, T, N, K, epi);
+    hipLaunchKernelGGL((seq_linear_kernel<P, NTD, TT, VEC, true>), dim3((N + NTD * 16 - 1) / (NTD * 16), grid.y, gz), dim3(256), 0,
+                       st, out, (const E*)x, (const E*)w, (const E*)bias, T, N, K, epi, ext);
   else
     hipLaunchKernelGGL((seq_linear_kernel<P, NT, TT, VEC, false>), grid, dim3(256), 0, st, out, (const E*)x, (const E*)w,
-                       (const E*)bias, T, N, K, epi);
+                       (const E*)bias, T, N, K, epi, ext);
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }
 
 template <typename P, bool VEC>
-static int launch_vec(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st) {
-  if (T <= 16) return launch_tt<P, 1, 1, VEC>(out, x, w, bias, T, N, K, epi, st);
-  if (T <= 32) return launch_tt<P, 1, 2, VEC>(out, x, w, bias, T, N, K, epi, st);
+static int launch_vec(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st,
+                      const LinExt& ext, int gz = 1) {
+  if (T <= 16) return launch_tt<P, 1, 1, VEC>(out, x, w, bias, T, N, K, epi, st, ext, 0, gz);
+  if (T <= 32) return launch_tt<P, 1, 2, VEC>(out, x, w, bias, T, N, K, epi, st, ext, 0, gz);
   // many tokens: the launch is bound by fragment loads per MFMA, not by weight bytes -> four output tiles per workgroup
   // (the K order of every output is unchanged: a row's value does not depend on which variant computed it)
+  const bool dense = gz == 1 && ext.ldx == K && ext.ldo == N && epi != EPI_GATE;
   if (T > 64 && N >= 64 && sizeof(typename El<P>::type) == 2) {
-    if (VEC && T >= 256 && N >= 128) return launch_wide<P>(out, x, w, bias, T, N, K, epi, st);      // both operands re-used
-    return launch_tt<P, 4, 4, VEC>(out, x, w, bias, T, N, K, epi, st);
+    if (VEC && dense && T >= 256 && N >= 128) return launch_wide<P>(out, x, w, bias, T, N, K, epi, st);      // both operands re-used
+    return launch_tt<P, 4, 4, VEC>(out, x, w, bias, T, N, K, epi, st, ext, 0, gz);
   }
-  return launch_tt<P, 1, 4, VEC>(out, x, w, bias, T, N, K, epi, st);
+  return launch_tt<P, 1, 4, VEC>(out, x, w, bias, T, N, K, epi, st, ext, 0, gz);
 }
 
 extern "C" int umb_seq_linear(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, int dtype,
@@ -320,8 +353,41 @@ extern "C" int umb_seq_linear(void* out, const void* x, const void* w, const voi
     if (N & 1) return UMB_EINVAL;
     N >>= 1;                                   // rows of each half
   }
+  const LinExt ext = lin_dense(N, K);
   DISPATCH_SEQ_DTYPE(dtype, {
-    if (K % 8 == 0) return launch_vec<P, true>(out, x, w, bias, T, N, K, epi, st);
-    return launch_vec<P, false>(out, x, w, bias, T, N, K, epi, st);
+    if (K % 8 == 0) return launch_vec<P, true>(out, x, w, bias, T, N, K, epi, st, ext);
+    return launch_vec<P, false>(out, x, w, bias, T, N, K, epi, st, ext);
+  })
+}
+
+extern "C" int umb_seq_linear_batched(void* out, const void* x, const void* w, int T, int N, int K, int ldx, int ldo, int batch,
+                                      long sx, long sw, long so, int epi, const float* gate, int ldg, int sg, int dtype,
+                                      hipStream_t st) {
+  if (T < 1 || N < 1 || K < 1 || batch < 1 || batch > 65535 || ldx < K || ldo < N || !out || !x || !w ||
+      !(epi == EPI_F32 || epi == EPI_DT || epi == EPI_GATE) || (epi == EPI_GATE && !gate))
+    return UMB_EINVAL;
+  const LinExt ext{ldx, ldo, sx, sw, so, 0, nullptr, gate, ldg, sg};
+  // 16-byte loads need every row start aligned: the strides as well as K
+  const bool vec = K % 8 == 0 && ldx % 8 == 0 && sx % 8 == 0 && sw % 8 == 0;
+  DISPATCH_SEQ_DTYPE(dtype, {
+    if (vec) return launch_vec<P, true>(out, x, w, nullptr, T, N, K, epi, st, ext, batch);
+    return launch_vec<P, false>(out, x, w, nullptr, T, N, K, epi, st, ext, batch);
+  })
+}
+
+extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, long gs, int N,
+                                      int K, int epi, int dtype, hipStream_t st) {
+  if (max_tiles < 1 || max_tiles > 65535 || N < 1 || K < 1 || epi < 0 || epi > 2 || !out || !x || !w || !tiles) return UMB_EINVAL;
+  if (epi == EPI_SILU_MUL) {
+    if (N & 1) return UMB_EINVAL;
+    N >>= 1;
+  }
+  const LinExt ext{K, N, 0, 0, 0, gs, tiles, nullptr, 0, 0};
+  DISPATCH_SEQ_DTYPE(dtype, {
+    if (K % 8 == 0 && gs % 8 == 0) {
+      if (N >= 64 && sizeof(typename El<P>::type) == 2) return launch_tt<P, 4, 4, true>(out, x, w, nullptr, 64, N, K, epi, st, ext, max_tiles);
+      return launch_tt<P, 1, 4, true>(out, x, w, nullptr, 64, N, K, epi, st, ext, max_tiles);
+    }
+    return launch_tt<P, 1, 4, false>(out, x, w, nullptr, 64, N, K, epi, st, ext, max_tiles);
   })
 }

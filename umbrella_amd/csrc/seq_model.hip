@@ -21,15 +21,67 @@ static inline int lin(const UmbSeqLinear& l, void* out, const void* x, int T, in
 
 static const void* first_norm_of(const UmbSeqModel* m, int l) { return l < m->L ? m->layers[l].norm1 : nullptr; }
 
+// What a sublayer reads.  With a pre-norm the seam kernel has already left norm(x) * w in ws->h.  Without one the sublayer
+// reads the residual stream itself through the causal convolution x + conv(x), whose last inputs are the sequence's state.
+static int sublayer_input(const UmbSeqModel* m, const UmbSeqWork* ws, const UmbSeqStep* s, const void* pre_norm, const void* canon,
+                          float* canon_state, hipStream_t st) {
+  const int T = s->T, W = m->W, dt = m->dtype;
+  if (pre_norm) return canon ? UMB_EINVAL : UMB_OK;           // a convolution on normed inputs is not implemented
+  if (!canon) return UMB_EINVAL;                              // every design so far has one of the two
+  if (s->max_len == 1) return umb_canon_step(ws->h, ws->x, canon, canon_state, s->pos, s->slot, T, W, m->canon_taps, dt, st);
+  SEQ_TRY(umb_canon_conv(ws->h, ws->x, canon, canon_state, s->pos, s->slot, T, W, m->canon_taps, dt, st));
+  return umb_canon_update(canon_state, ws->x, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B, W, m->canon_taps, st);
+}
+
+// feed-forward of ws->h into ws->y (fp32)
+static int feed_forward(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSeqWork* ws, const UmbSeqStep* s, hipStream_t st) {
+  const int T = s->T, W = m->W, dt = m->dtype;
+  if (ly.ff_kind == UMB_FF_GATED) {
+    SEQ_TRY(lin(ly.gu, ws->act, ws->h, T, 2, dt, st));
+    return lin(ly.down, ws->y, ws->act, T, 0, dt, st);
+  }
+  if (ly.ff_kind == UMB_FF_POLYNORM) {
+    if (!ly.act || ly.gu.N != ly.ff) return UMB_EINVAL;
+    SEQ_TRY(lin(ly.gu, ws->proj, ws->h, T, 0, dt, st));                        // "up" alone
+    SEQ_TRY(umb_polynorm(ws->act, ws->proj, ly.act, T, ly.ff, m->eps, dt, st));
+    return lin(ly.down, ws->y, ws->act, T, 0, dt, st);
+  }
+  if (ly.ff_kind == UMB_FF_MOE) {
+    const int E = ly.experts, top = ly.top, F = ly.expert_ff;
+    if (E < 1 || top < 1 || top > E || F < 1 || !ly.e_gu || !ly.e_down || !ws->moe_sel || !ws->moe_wt || !ws->moe_pos ||
+        !ws->moe_tiles || !ws->moe_xs || !ws->moe_act || !ws->moe_y || ly.router.N != E)
+      return UMB_EINVAL;
+    const long pairs = (long)T * top;
+    const int max_tiles = (int)((pairs + 63) / 64) + E;
+    if (max_tiles > ws->moe_max_tiles) return UMB_EINVAL;
+    if (ly.s_gu.w) {                                                           // the shared expert sees every token
+      SEQ_TRY(lin(ly.s_gu, ws->act, ws->h, T, 2, dt, st));
+      SEQ_TRY(lin(ly.s_down, ws->y, ws->act, T, 0, dt, st));
+    }
+    SEQ_TRY(lin(ly.router, ws->proj, ws->h, T, 0, dt, st));
+    SEQ_TRY(umb_moe_route(ws->moe_sel, ws->moe_wt, ws->proj, T, E, top, st));
+    SEQ_TRY(umb_moe_plan(ws->moe_pos, ws->moe_tiles, ws->moe_sel, T, E, top, max_tiles, st));
+    SEQ_TRY(umb_moe_scatter(ws->moe_xs, ws->h, ws->moe_wt, ws->moe_pos, T, W, top, dt, st));
+    SEQ_TRY(umb_seq_linear_grouped(ws->moe_act, ws->moe_xs, ly.e_gu, ws->moe_tiles, max_tiles, 2L * F * W, 2 * F, W, 2, dt, st));
+    SEQ_TRY(umb_seq_linear_grouped(ws->moe_y, ws->moe_act, ly.e_down, ws->moe_tiles, max_tiles, (long)W * F, W, F, 0, dt, st));
+    return umb_moe_combine(ws->y, ws->moe_y, ws->moe_pos, T, W, top, ly.s_gu.w ? 1 : 0, st);
+  }
+  return UMB_EINVAL;
+}
+
 extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const UmbSeqStep* s, hipStream_t st) {
   if (!m || !ws || !s || m->L < 1 || !m->layers || s->T < 1 || s->T > ws->Tmax || s->B < 1 || s->R < 0 || s->R > ws->Rmax)
     return UMB_EINVAL;
   const int T = s->T, W = m->W, dt = m->dtype, groups = m->groups;
   const float eps = m->eps;
-  SEQ_TRY(umb_seq_embed_norm(ws->x, ws->h, m->embed, s->tokens, m->layers[0].norm1, T, W, m->V, groups, eps, dt, st));
+  if (m->layers[0].norm1)
+    SEQ_TRY(umb_seq_embed_norm(ws->x, ws->h, m->embed, s->tokens, m->layers[0].norm1, T, W, m->V, groups, eps, dt, st));
+  else
+    SEQ_TRY(umb_seq_embed(ws->x, m->embed, s->tokens, m->embed_scale, T, W, m->V, dt, st));
   for (int l = 0; l < m->L; ++l) {
     const UmbSeqLayer& ly = m->layers[l];
     const int ld = ly.proj.N;
+    SEQ_TRY(sublayer_input(m, ws, s, ly.norm1, ly.canon1, ly.canon_state1, st));
     SEQ_TRY(lin(ly.proj, ws->proj, ws->h, T, 0, dt, st));
     if (ly.kind == UMB_MIX_POOLED_WINDOW) {
       const int H = ly.heads, G = ly.kv_heads, D = ly.dim;
@@ -50,6 +102,26 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
       SEQ_TRY(umb_gla_scan(ws->o, ly.state, ws->proj, ld, ws->aux, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B, H, D,
                            Dv, ly.qscale, st));
       SEQ_TRY(umb_gla_gate(ws->mix, ws->o, ws->proj, ld, 2 * HD + H * Dv, ly.head_norm, T, H, Dv, eps, dt, st));
+    } else if (ly.kind == UMB_MIX_LATENT) {
+      // proj = [dq | dkv (latent + rotated key part) | gate]; the query latent goes up to the heads, its unrotated parts are
+      // carried into the key/value latent space (W_uk^T, one product per head), attention runs against the cached rows, the
+      // value up-projection W_uv follows the weighted sum, with the sigmoid gate as its epilogue
+      const int H = ly.heads, D = ly.dim, R = ly.rot_dim, Dv = ly.vdim, Rq = ly.q_rank, Rc = ly.kv_rank, Dk = Rc + R;
+      if (ld != Rq + Dk + H * Dv || ly.uq.N != H * (D + R) || ly.uq.K != Rq || !ly.uk_t || !ly.uv || !ly.dq_norm || !ly.dkv_norm)
+        return UMB_EINVAL;
+      SEQ_TRY(umb_lat_prep(ws->act, &ly.kv, ws->proj, ld, ly.dq_norm, ly.dkv_norm, s->pos, s->slot, ly.rot_freq, T, Rq, Rc, R,
+                           ly.rot_dims, eps, dt, st));
+      SEQ_TRY(lin(ly.uq, ws->o, ws->act, T, 0, dt, st));
+      SEQ_TRY(umb_lat_qsplit(ws->mix, ws->aux, ws->o, s->pos, ly.rot_freq, T, H, D, R, Rc, ly.rot_dims, dt, st));
+      SEQ_TRY(umb_seq_linear_batched(ws->aux, ws->mix, ly.uk_t, T, Rc, D, H * D, H * Dk, H, D, (long)Rc * D, Dk, 0, nullptr, 0, 0,
+                                     dt, st));
+      if (s->max_len >= 16 && umb_lat_attend_tiled_ok(H, Rc, R, dt))
+        SEQ_TRY(umb_lat_attend_tiled(ws->act, ws->aux, &ly.kv, ly.sink, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B,
+                                     s->max_len, H, Rc, R, ly.window, ly.scale, dt, st));
+      else
+        SEQ_TRY(umb_lat_attend(ws->act, ws->aux, &ly.kv, ly.sink, s->pos, s->slot, T, H, Rc, R, ly.window, ly.scale, dt, st));
+      SEQ_TRY(umb_seq_linear_batched(ws->mix, ws->act, ly.uv, T, Dv, Rc, H * Rc, H * Dv, H, Rc, (long)Dv * Rc, Dv, 3,
+                                     ws->proj + Rq + Dk, ld, Dv, dt, st));
     } else {
       return UMB_EINVAL;
     }
@@ -57,8 +129,8 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
     const void* next = ly.has_mlp ? ly.norm2 : first_norm_of(m, l + 1);
     SEQ_TRY(umb_seq_resid_norm(ws->x, ws->h, ws->y, ly.norm1b, next, T, W, groups, eps, dt, st));
     if (ly.has_mlp) {
-      SEQ_TRY(lin(ly.gu, ws->act, ws->h, T, 2, dt, st));
-      SEQ_TRY(lin(ly.down, ws->y, ws->act, T, 0, dt, st));
+      SEQ_TRY(sublayer_input(m, ws, s, ly.norm2, ly.canon2, ly.canon_state2, st));
+      SEQ_TRY(feed_forward(m, ly, ws, s, st));
       SEQ_TRY(umb_seq_resid_norm(ws->x, ws->h, ws->y, ly.norm2b, first_norm_of(m, l + 1), T, W, groups, eps, dt, st));
     }
     if (s->trace) {

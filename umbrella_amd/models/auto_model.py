@@ -12,6 +12,7 @@ from __future__ import annotations
 import os
 
 from .config import KNOWN, read_architecture
+from .fidizen import Fidizen
 from .gitopel import Gitopel
 from .llama import Llama
 
@@ -19,7 +20,7 @@ from .llama import Llama
 class AutoModelLM:
     # a local directory is resolved by the architecture its config.json names; directories that name none of these are
     # Hugging Face Llama / Qwen2 / Mistral checkpoints
-    _ARCHITECTURE_MAPPING = {"Gitopel": Gitopel}
+    _ARCHITECTURE_MAPPING = {"Gitopel": Gitopel, "Fidizen": Fidizen}
     _MODEL_MAPPING = {name: Llama for name in KNOWN}
     _OFFLOAD_MODEL_MAPPING = dict(_MODEL_MAPPING)
     _CUDAGRAPH_MODEL_MAPPING = dict(_MODEL_MAPPING)

@@ -222,9 +222,39 @@ class GLACfg:
 
 
 @dataclass
+class LatentAttnCfg:
+    """Softmax attention through low-rank latents: queries via a normed latent of ``q_rank``, keys / values via a normed
+    latent of ``kv_rank`` (the only thing cached, with one rotated key part of ``rot_dim`` shared by the heads); per head
+    ``dim`` unrotated + ``rot_dim`` rotated query / key features and ``vdim`` value features; interleaved rotary on the
+    first ``rot_dims`` of the rotated part; sliding window (0: none); a sink per head in the softmax denominator; a
+    sigmoid output gate."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    window: int
+    rot_dims: int
+    rot_base: float
+    scale: float
+    kind: str = "latent_attention"
+
+
+@dataclass
 class SeqLayerCfg:
-    mixer: object                    # PooledWindowAttnCfg | GLACfg
-    ff: int = 0                      # width of the gated feed-forward; 0 = the layer has none
+    mixer: object                    # PooledWindowAttnCfg | GLACfg | LatentAttnCfg
+    ff: int = 0                      # width of the dense feed-forward; 0 = the layer has none (or has experts)
+    ff_kind: str = "gated"           # "gated": W_down (silu(W_gate h) * W_up h); "polynorm": W_down polynorm(W_up h); "moe"
+    experts: int = 0                 # "moe": routed experts, how many each token uses, their width, the shared expert's
+    top: int = 0
+    expert_ff: int = 0
+    shared_ff: int = 0               # 0: no shared expert
+    weights_of: int | None = None    # the layer uses that layer's tensors (with a cache and state of its own)
+
+    @property
+    def has_ff(self) -> bool:
+        return self.ff > 0 or self.ff_kind == "moe"
 
 
 @dataclass
@@ -237,6 +267,9 @@ class SeqMixCfg:
     name: str = "seqmix"
     architecture: str = ""
     eos_token_id: list = field(default_factory=list)
+    embed_scale: float = 1.0         # the embedding row is multiplied by it
+    pre_norm: bool = True            # False: sublayers read the residual stream itself, only their output is normed
+    canon_taps: int = 0              # > 0: every sublayer reads h + causal_conv(h) over this many positions (pre_norm False)
 
     @property
     def num_hidden_layers(self):

@@ -24,7 +24,8 @@ from ..attn.cache import PagedSeqCache
 from .base import LLMBase
 from .config import SeqMixCfg
 
-KIND_CODE = {"attention": 0, "gla": 1}
+KIND_CODE = {"attention": 0, "gla": 1, "latent_attention": 2}
+FF_CODE = {"gated": 0, "polynorm": 1, "moe": 2}
 
 
 def _linear(w, b=None) -> UmbSeqLinear:
@@ -93,10 +94,16 @@ class SeqMixLM(LLMBase):
         self._top = self.top_tensors(get)
         assert tuple(self._top["embed"].shape) == (c.vocab_size, c.width), tuple(self._top["embed"].shape)
         L = len(c.layers)
-        self._tensors, kv_layers, state_layers = [], [], []
+        self._tensors, kv_layers, state_layers, latent_layers, n_conv = [], [], [], [], 0
         for i, ly in enumerate(c.layers):
-            t = self.layer_tensors(i, ly, get)
-            t = {k: (v.contiguous() if isinstance(v, torch.Tensor) else v) for k, v in t.items()}
+            if ly.weights_of is not None:
+                # the tensors of another layer (which must own its tensors), a cache and state of this layer's own
+                if not (0 <= ly.weights_of < i) or c.layers[ly.weights_of].weights_of is not None:
+                    raise ValueError(f"layer {i}: weights_of must name an earlier layer that has tensors of its own")
+                t = dict(self._tensors[ly.weights_of])
+            else:
+                t = self.layer_tensors(i, ly, get)
+                t = {k: (v.contiguous() if isinstance(v, torch.Tensor) else v) for k, v in t.items()}
             m = ly.mixer
             if m.kind == "attention":
                 if m.vdim != m.dim:
@@ -105,33 +112,65 @@ class SeqMixLM(LLMBase):
                     raise ValueError("heads must be a multiple of kv_heads")
                 t["cache_index"] = len(kv_layers)
                 kv_layers.append((m.kv_heads, m.dim, m.pool))
-                i2 = torch.arange(m.rot_dims // 2, dtype=torch.float32)
-                t["rot_freq"] = (m.rot_base ** (-2 * i2 / m.rot_dims)).to(dev) if m.rot_dims else None     # fp32 frequencies
+            elif m.kind == "latent_attention":
+                t["cache_index"] = len(latent_layers)
+                latent_layers.append(m.kv_rank + m.rot_dim)
             else:
                 t["cache_index"] = len(state_layers)
                 state_layers.append((m.heads, m.dim, m.vdim))
+            if m.kind != "gla" and "rot_freq" not in t:
+                i2 = torch.arange(m.rot_dims // 2, dtype=torch.float32)
+                t["rot_freq"] = (m.rot_base ** (-2 * i2 / m.rot_dims)).to(dev) if m.rot_dims else None     # fp32 frequencies
+            if c.canon_taps > 0:
+                t["conv_index"] = n_conv
+                n_conv += 2 if ly.has_ff else 1
             self._tensors.append(t)
-        self.kv_cache = PagedSeqCache(kv_layers, state_layers, self.max_tokens, self.batch_size, dev, dt, page=self.page_size)
+        self.kv_cache = PagedSeqCache(kv_layers, state_layers, self.max_tokens, self.batch_size, dev, dt, page=self.page_size,
+                                      latent_layers=latent_layers, conv_states=n_conv, conv_taps=c.canon_taps, width=c.width)
         self._layer_structs = (UmbSeqLayer * L)()
         for i, (ly, t) in enumerate(zip(c.layers, self._tensors)):
             s, m = self._layer_structs[i], ly.mixer
-            s.kind, s.has_mlp, s.heads, s.dim, s.vdim, s.ff = KIND_CODE[m.kind], int(ly.ff > 0), m.heads, m.dim, m.vdim, ly.ff
-            s.proj, s.out = _linear(t["proj_w"], t["proj_b"]), _linear(t["out_w"], t["out_b"])
-            s.norm1, s.norm1b = t["norm1"].data_ptr(), t["norm1b"].data_ptr()
+            s.kind, s.has_mlp, s.heads, s.dim, s.vdim, s.ff = KIND_CODE[m.kind], int(ly.has_ff), m.heads, m.dim, m.vdim, ly.ff
+            s.ff_kind = FF_CODE[ly.ff_kind]
+            s.proj, s.out = _linear(t["proj_w"], t.get("proj_b")), _linear(t["out_w"], t.get("out_b"))
+            s.norm1 = t["norm1"].data_ptr() if t.get("norm1") is not None else None
+            s.norm1b = t["norm1b"].data_ptr()
+            if c.canon_taps > 0:
+                s.canon1, s.canon_state1 = t["canon1"].data_ptr(), self.kv_cache.conv[t["conv_index"]].data_ptr()
             if m.kind == "attention":
                 s.kv_heads, s.window, s.pool, s.rot_dims, s.scale = m.kv_heads, m.window, m.pool, m.rot_dims, m.scale
                 s.pos_bias = t["pos_bias"].data_ptr() if t.get("pos_bias") is not None else None
                 s.rot_freq = t["rot_freq"].data_ptr() if t["rot_freq"] is not None else None
                 s.kv = self.kv_cache.struct(t["cache_index"])
+            elif m.kind == "latent_attention":
+                s.q_rank, s.kv_rank, s.rot_dim, s.rot_dims, s.scale = m.q_rank, m.kv_rank, m.rot_dim, m.rot_dims, m.scale
+                s.window = m.window if m.window > 0 else 2 ** 30            # no window: every earlier position is seen
+                s.rot_freq = t["rot_freq"].data_ptr() if t["rot_freq"] is not None else None
+                s.uq, s.uk_t, s.uv = _linear(t["uq_w"]), t["uk_t"].data_ptr(), t["uv_w"].data_ptr()
+                s.dq_norm, s.dkv_norm = t["dq_norm"].data_ptr(), t["dkv_norm"].data_ptr()
+                s.sink = t["sink"].data_ptr() if t.get("sink") is not None else None
+                s.kv = self.kv_cache.latent_struct(t["cache_index"])
             else:
                 s.rank, s.tau, s.qscale = m.rank, m.tau, float(m.dim) ** -0.5
                 s.a2, s.head_norm = _linear(t["a2_w"], t["a2_b"]), t["head_norm"].data_ptr()
                 s.state = self.kv_cache.state[t["cache_index"]].data_ptr()
-            if ly.ff:
-                s.norm2, s.norm2b = t["norm2"].data_ptr(), t["norm2b"].data_ptr()
-                s.gu, s.down = _linear(t["gu_w"]), _linear(t["down_w"])
+            if ly.has_ff:
+                s.norm2 = t["norm2"].data_ptr() if t.get("norm2") is not None else None
+                s.norm2b = t["norm2b"].data_ptr()
+                if c.canon_taps > 0:
+                    s.canon2, s.canon_state2 = t["canon2"].data_ptr(), self.kv_cache.conv[t["conv_index"] + 1].data_ptr()
+                if ly.ff_kind == "moe":
+                    s.experts, s.top, s.expert_ff, s.shared_ff = ly.experts, ly.top, ly.expert_ff, ly.shared_ff
+                    s.router, s.e_gu, s.e_down = _linear(t["router_w"]), t["e_gu"].data_ptr(), t["e_down"].data_ptr()
+                    if ly.shared_ff:
+                        s.s_gu, s.s_down = _linear(t["s_gu_w"]), _linear(t["s_down_w"])
+                else:
+                    s.gu, s.down = _linear(t["gu_w"]), _linear(t["down_w"])      # polynorm: gu is the up-projection alone
+                    if ly.ff_kind == "polynorm":
+                        s.act = t["act"].data_ptr()
         mdl = self._m = UmbSeqModel()
         mdl.dtype, mdl.L, mdl.W, mdl.V, mdl.groups, mdl.eps = _lib.seq_dtype_code(dt), L, c.width, c.vocab_size, c.norm_groups, c.norm_eps
+        mdl.embed_scale, mdl.canon_taps = float(c.embed_scale), int(c.canon_taps)
         mdl.embed, mdl.final_norm, mdl.head = self._top["embed"].data_ptr(), self._top["final_norm"].data_ptr(), _linear(self._top["head"])
         mdl.layers = C.cast(self._layer_structs, C.POINTER(UmbSeqLayer))
         self.reserve(self.max_step_tokens or 256)
@@ -146,20 +185,48 @@ class SeqMixLM(LLMBase):
         T, R = max(tokens, self.ws_tokens), max(logit_rows, self.logit_rows)
         self._graphs = {}                               # captured steps hold the old workspace's addresses
         c, dev, dt = self.config, self.device, self.dtype
-        projN = max(t["proj_w"].shape[0] for t in self._tensors)
-        hd = max(ly.mixer.heads * ly.mixer.dim for ly in c.layers)
-        hv = max(ly.mixer.heads * ly.mixer.vdim for ly in c.layers)
-        ff = max([ly.ff for ly in c.layers] + [1])
-        f32 = torch.float32
+        # widths of the shared scratch buffers: the largest any layer asks of each
+        need = dict(proj=1, aux=1, o=1, mix=1, act=1)
+
+        def ask(**kw):
+            for k, v in kw.items():
+                need[k] = max(need[k], int(v))
+        top = eff = 0
+        for ly, t in zip(c.layers, self._tensors):
+            m = ly.mixer
+            ask(proj=t["proj_w"].shape[0])
+            if m.kind == "latent_attention":
+                # act: query latent, then the attended latents; o: queries; mix: unrotated queries, then the gated heads;
+                # aux: queries carried into the latent space
+                ask(act=max(m.q_rank, m.heads * m.kv_rank), o=m.heads * (m.dim + m.rot_dim), mix=m.heads * max(m.dim, m.vdim),
+                    aux=m.heads * (m.kv_rank + m.rot_dim))
+            else:
+                ask(aux=m.heads * m.dim, o=m.heads * m.vdim, mix=m.heads * m.vdim)
+            if ly.ff_kind == "moe":
+                ask(proj=ly.experts, act=ly.shared_ff)
+                top, eff = max(top, ly.top), max(eff, ly.expert_ff)
+            elif ly.ff:
+                ask(act=ly.ff, proj=ly.ff if ly.ff_kind == "polynorm" else 1)
+        f32, i32 = torch.float32, torch.int32
         b = self._bufs = dict(
             x=torch.zeros(T, c.width, dtype=f32, device=dev), h=torch.zeros(T, c.width, dtype=dt, device=dev),
-            proj=torch.zeros(T, projN, dtype=f32, device=dev), aux=torch.zeros(T, hd, dtype=f32, device=dev),
-            o=torch.zeros(T, hv, dtype=f32, device=dev), mix=torch.zeros(T, hv, dtype=dt, device=dev),
-            act=torch.zeros(T, ff, dtype=dt, device=dev), y=torch.zeros(T, c.width, dtype=f32, device=dev),
+            proj=torch.zeros(T, need["proj"], dtype=f32, device=dev), aux=torch.zeros(T, need["aux"], dtype=f32, device=dev),
+            o=torch.zeros(T, need["o"], dtype=f32, device=dev), mix=torch.zeros(T, need["mix"], dtype=dt, device=dev),
+            act=torch.zeros(T, need["act"], dtype=dt, device=dev), y=torch.zeros(T, c.width, dtype=f32, device=dev),
             logits=torch.zeros(R, c.vocab_size, dtype=f32, device=dev))
         ws = self._ws = UmbSeqWork()
         for k in ("x", "h", "proj", "aux", "o", "mix", "act", "y", "logits"):
             setattr(ws, k, b[k].data_ptr())
+        if top:
+            pairs = T * top
+            tiles = (pairs + 63) // 64 + max(ly.experts for ly in c.layers)
+            b.update(moe_sel=torch.zeros(pairs, dtype=i32, device=dev), moe_wt=torch.zeros(pairs, dtype=f32, device=dev),
+                     moe_pos=torch.zeros(pairs, dtype=i32, device=dev), moe_tiles=torch.zeros(tiles, 3, dtype=i32, device=dev),
+                     moe_xs=torch.zeros(pairs, c.width, dtype=dt, device=dev), moe_act=torch.zeros(pairs, eff, dtype=dt, device=dev),
+                     moe_y=torch.zeros(pairs, c.width, dtype=f32, device=dev))
+            for k in ("moe_sel", "moe_wt", "moe_pos", "moe_tiles", "moe_xs", "moe_act", "moe_y"):
+                setattr(ws, k, b[k].data_ptr())
+            ws.moe_max_tiles = tiles
         ws.Tmax, ws.Rmax = T, R
         self.ws_tokens, self.logit_rows = T, R
 
@@ -259,5 +326,6 @@ class SeqMixLM(LLMBase):
         return self.inference(input_ids, position_ids, attention_mask, storage_ids)
 
     def weight_bytes(self) -> int:
-        n = sum(v.numel() * v.element_size() for t in self._tensors for v in t.values() if isinstance(v, torch.Tensor))
+        n = sum(v.numel() * v.element_size() for ly, t in zip(self.config.layers, self._tensors) if ly.weights_of is None
+                for v in t.values() if isinstance(v, torch.Tensor))
         return n + self._top["head"].numel() * self._top["head"].element_size()
