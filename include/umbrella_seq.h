@@ -85,8 +85,9 @@ int umb_canon_step(void* h, const float* x, const void* w, float* state, const i
  * N(v) = v / sqrt(mean(v^2) + eps) over the row; coef = {a, b, c, e} in `dtype`; z fp32 [T][F], out in `dtype`. */
 int umb_polynorm(void* out, const float* z, const void* coef, int T, int F, float eps, int dtype, umb_stream_t stream);
 
-/* ---- routed experts.  logits fp32 [T][E]; scores = sigmoid(logits); each token keeps its `top` largest (ties: the lower
- * index), weight = the score itself.  sel [T][top] expert ids, wt [T][top] fp32. */
+/* ---- routed experts.  logits fp32 [T][E]; scores = sigmoid(logits); each token keeps its `top` largest (compared on the
+ * logits, so scores that saturate to the same fp32 value are still told apart; ties: the lower index), weight = the score
+ * itself.  sel [T][top] expert ids, wt [T][top] fp32. */
 int umb_moe_route(int* sel, float* wt, const float* logits, int T, int E, int top, umb_stream_t stream);
 /* orders the T*top (token, choice) pairs by expert: pos_of [T*top] = row of the pair in the expert-ordered list,
  * tiles [max_tiles][3] = {expert, first row, rows} covering every expert's rows in pieces of at most 64

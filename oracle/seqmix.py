@@ -133,3 +133,103 @@ def gitopel_forward(cfg: dict, sd: dict, tokens, dtype=F, cache_round=None, laye
         if layers_out is not None:
             layers_out.append(x.clone())
     return group_rms_norm(x, w["final.norm"], groups, eps) @ w["head"].T
+
+
+# ---------------------------------------------------------------------------------------------------------------- Fidizen
+def rms_norm(x, w, eps: float):
+    return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w
+
+
+def conv_input(h, w, history=None):
+    """What a sublayer reads: h[t] + sum_j w[:, j] * h[t - taps + 1 + j] (j = taps - 1 is h[t] itself), zeros before the
+    start.  h [n, width], w [width, taps]; history: the inputs that came before h[0] (any number of rows, the last is
+    h[-1])."""
+    taps, n = w.shape[1], h.shape[0]
+    past = torch.zeros(0, h.shape[1], dtype=h.dtype) if history is None else history
+    full = torch.cat([past, h])
+    off = past.shape[0]
+    out = h.clone()
+    for t in range(n):
+        for j in range(taps):
+            src = off + t - taps + 1 + j
+            if src >= 0:
+                out[t] = out[t] + w[:, j] * full[src]
+    return out
+
+
+def latent_attention(X, w_dq, n_dq, w_uq, w_dkv, n_dkv, w_uk, w_uv, sink, w_g, w_o, *, H, D, R, E, kv_rank, window, rot_dims,
+                     base, scale, eps, cache_round=None, pos0: int = 0):
+    """Softmax attention through latents.  c_q = norm(w_dq x), q = w_uq c_q laid out per head as [D unrotated | R rotated];
+    w_dkv x = [kv_rank latent | R shared key part]; c = norm(latent); per head key = [w_uk c | rotated shared part], value =
+    w_uv c.  Position i sees j with 0 <= i - j < window (window 0: all j <= i).  The softmax denominator also holds
+    exp(sink[h]).  The heads, concatenated, are multiplied by sigmoid(w_g x) and go through w_o.
+    cache_round: optional rounding of what a cache would hold (c and the rotated shared key part)."""
+    n = X.shape[0]
+    pos = torch.arange(pos0, pos0 + n)
+    q = (rms_norm(X @ w_dq.T, n_dq, eps) @ w_uq.T).reshape(n, H, D + R)
+    q_rot = rotate_interleaved(q[..., D:], pos, rot_dims, base)
+    dkv = X @ w_dkv.T
+    c = rms_norm(dkv[:, :kv_rank], n_dkv, eps)
+    k_rot = rotate_interleaved(dkv[:, None, kv_rank:], pos, rot_dims, base)[:, 0]
+    if cache_round is not None:
+        c, k_rot = cache_round(c), cache_round(k_rot)
+    k = (c @ w_uk.T).reshape(n, H, D)
+    v = (c @ w_uv.T).reshape(n, H, E)
+    out = torch.zeros(n, H, E, dtype=X.dtype)
+    for t in range(n):
+        lo = 0 if window <= 0 else max(0, t - window + 1)
+        for h in range(H):
+            s = (k[lo:t + 1, h] @ q[t, h, :D] + k_rot[lo:t + 1] @ q_rot[t, h]) * scale          # one score per visible j
+            m = torch.maximum(s.max(), sink[h])
+            e = torch.exp(s - m)
+            p = e / (e.sum() + torch.exp(sink[h] - m))
+            out[t, h] = (p[:, None] * v[lo:t + 1, h]).sum(0)
+    return (out.reshape(n, H * E) * torch.sigmoid(X @ w_g.T)) @ w_o.T
+
+
+def polynorm(z, coef, eps: float):
+    """coef[0] N(z) + coef[1] N(z^2) + coef[2] N(z^3) + coef[3], N = unit RMS over the row"""
+    return coef[0] * unit_rms(z, eps) + coef[1] * unit_rms(z * z, eps) + coef[2] * unit_rms(z * z * z, eps) + coef[3]
+
+
+def routed_experts(X, w_router, experts, top: int, shared=None):
+    """experts: list of (w_gate, w_up, w_down).  score = sigmoid(router logit); the `top` largest (ties: lower index) are
+    used, each expert fed score * x; outputs summed; `shared` (same triple) sees every token unweighted."""
+    s = torch.sigmoid(X @ w_router.T)
+    out = torch.zeros_like(X)
+    for t in range(X.shape[0]):
+        order = sorted(range(len(experts)), key=lambda e: (-float(s[t, e]), e))[:top]
+        for e in order:
+            out[t] = out[t] + gated_ff((s[t, e] * X[t])[None], *experts[e])[0]
+    if shared is not None:
+        out = out + gated_ff(X, *shared)
+    return out
+
+
+def fidizen_forward(cfg: dict, sd: dict, tokens, dtype=F, cache_round=None, layers_out=None):
+    """Whole-sequence forward of a Fidizen checkpoint: cfg is the parsed config.json, sd maps tensor names to tensors.
+    Returns logits [n, vocab]."""
+    w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in sd.items()}
+    eps = cfg["norm"]["eps"]
+    x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * cfg["embedding"]["scale"]
+    for i, ly in enumerate(cfg["layers"]):
+        p, m = f"l{ly.get('weights_of', i) if ly.get('weights_of') is not None else i}.", ly["mixer"]
+        h = conv_input(x, w[p + "canon1"])
+        y = latent_attention(h, w[p + "mix.dq"], w[p + "mix.dq.norm"], w[p + "mix.uq"], w[p + "mix.dkv"], w[p + "mix.dkv.norm"],
+                             w[p + "mix.uk"], w[p + "mix.uv"], w[p + "mix.sink"], w[p + "mix.g"], w[p + "mix.o"], H=m["heads"],
+                             D=m["dim"], R=m["rot_dim"], E=m["vdim"], kv_rank=m["kv_rank"], window=(m.get("mask") or {}).get("size", 0),
+                             rot_dims=m["rot"]["dims"], base=m["rot"]["base"], scale=m["scale"], eps=eps, cache_round=cache_round)
+        x = x + rms_norm(y, w[p + "norm1"], eps)
+        mlp = ly.get("mlp")
+        if mlp is not None:
+            h = conv_input(x, w[p + "canon2"])
+            if mlp["kind"] == "dense":
+                y = polynorm(h @ w[p + "mlp.up"].T, w[p + "mlp.act"], eps) @ w[p + "mlp.down"].T
+            else:
+                ex = [tuple(w[p + f"mlp.e{e}.{n}"] for n in ("gate", "up", "down")) for e in range(mlp["router"]["experts"])]
+                sh = tuple(w[p + f"mlp.shared.{n}"] for n in ("gate", "up", "down")) if mlp.get("shared") else None
+                y = routed_experts(h, w[p + "mlp.router"], ex, mlp["router"]["top"], sh)
+            x = x + rms_norm(y, w[p + "norm2"], eps)
+        if layers_out is not None:
+            layers_out.append(x.clone())
+    return rms_norm(x, w["final.norm"], eps) @ w["head"].T

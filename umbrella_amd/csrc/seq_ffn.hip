@@ -38,7 +38,9 @@ __global__ __launch_bounds__(256) void polynorm_kernel(typename El<P>::type* __r
   }
 }
 
-// one wave per token; lane l looks at experts l, l + 64, ...; `top` rounds of arg-max over the scores not yet taken
+// one wave per token; lane l looks at experts l, l + 64, ...; `top` rounds of arg-max over the experts not yet taken.  The
+// order is taken on the logits: the sigmoid is monotonic, and where it saturates in fp32 (two scores both rounding to 1) the
+// logits still tell the experts apart.
 __global__ __launch_bounds__(256) void moe_route_kernel(int* __restrict__ sel, float* __restrict__ wt,
                                                         const float* __restrict__ logits, int T, int E, int top) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -46,15 +48,15 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int* __restrict__ sel, f
   if (t >= T) return;
   const float* z = logits + (long)t * E;
   int prev_i = -1;
-  float prev_s = INFINITY;
+  float prev_z = INFINITY;
   for (int k = 0; k < top; ++k) {
-    // candidates come after (prev_s, prev_i) in the order "score descending, index ascending"
-    float best = -1.f;
+    // candidates come after (prev_z, prev_i) in the order "logit descending, index ascending"
+    float best = -INFINITY;
     int bi = 0x7fffffff;
     for (int e = lane; e < E; e += 64) {
-      const float s = 1.f / (1.f + expf(-z[e]));
-      const bool after = s < prev_s || (s == prev_s && e > prev_i);
-      if (after && (s > best || (s == best && e < bi))) { best = s; bi = e; }
+      const float v = z[e];
+      const bool after = v < prev_z || (v == prev_z && e > prev_i);
+      if (after && (v > best || (v == best && e < bi))) { best = v; bi = e; }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -62,9 +64,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int* __restrict__ sel, f
       const int oi = __shfl_xor(bi, o, 64);
       if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
     }
-    if (bi >= E) { bi = 0; best = 0.f; }            // no candidate left (scores that are not numbers): keep indices in range
-    if (lane == 0) { sel[(long)t * top + k] = bi; wt[(long)t * top + k] = best; }
-    prev_s = best; prev_i = bi;
+    if (bi >= E) { bi = 0; best = -INFINITY; }      // no candidate left (logits that are not numbers): keep indices in range
+    if (lane == 0) { sel[(long)t * top + k] = bi; wt[(long)t * top + k] = 1.f / (1.f + expf(-best)); }
+    prev_z = best; prev_i = bi;
   }
 }
 
