@@ -192,13 +192,19 @@ def polynorm(z, coef, eps: float):
     return coef[0] * unit_rms(z, eps) + coef[1] * unit_rms(z * z, eps) + coef[2] * unit_rms(z * z * z, eps) + coef[3]
 
 
-def routed_experts(X, w_router, experts, top: int, shared=None):
+def routed_experts(X, w_router, experts, top: int, shared=None, margins=None):
     """experts: list of (w_gate, w_up, w_down).  score = sigmoid(router logit); the `top` largest (ties: lower index) are
-    used, each expert fed score * x; outputs summed; `shared` (same triple) sees every token unweighted."""
-    s = torch.sigmoid(X @ w_router.T)
+    used, each expert fed score * x; outputs summed; `shared` (same triple) sees every token unweighted.
+    margins: optional list that receives, per token, how far the last chosen logit lies above the first one not chosen, in
+    units of the spread of that token's logits (tests pick inputs whose choices no rounding can flip)."""
+    z = X @ w_router.T
+    s = torch.sigmoid(z)
     out = torch.zeros_like(X)
     for t in range(X.shape[0]):
-        order = sorted(range(len(experts)), key=lambda e: (-float(s[t, e]), e))[:top]
+        ranked = sorted(range(len(experts)), key=lambda e: (-float(s[t, e]), e))
+        order = ranked[:top]
+        if margins is not None and top < len(experts):
+            margins.append(float((z[t, ranked[top - 1]] - z[t, ranked[top]]) / z[t].std().clamp_min(1e-30)))
         for e in order:
             out[t] = out[t] + gated_ff((s[t, e] * X[t])[None], *experts[e])[0]
     if shared is not None:
@@ -206,9 +212,9 @@ def routed_experts(X, w_router, experts, top: int, shared=None):
     return out
 
 
-def fidizen_forward(cfg: dict, sd: dict, tokens, dtype=F, cache_round=None, layers_out=None):
+def fidizen_forward(cfg: dict, sd: dict, tokens, dtype=F, cache_round=None, layers_out=None, route_margins=None):
     """Whole-sequence forward of a Fidizen checkpoint: cfg is the parsed config.json, sd maps tensor names to tensors.
-    Returns logits [n, vocab]."""
+    Returns logits [n, vocab].  route_margins: see routed_experts."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in sd.items()}
     eps = cfg["norm"]["eps"]
     x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * cfg["embedding"]["scale"]
@@ -228,7 +234,7 @@ def fidizen_forward(cfg: dict, sd: dict, tokens, dtype=F, cache_round=None, laye
             else:
                 ex = [tuple(w[p + f"mlp.e{e}.{n}"] for n in ("gate", "up", "down")) for e in range(mlp["router"]["experts"])]
                 sh = tuple(w[p + f"mlp.shared.{n}"] for n in ("gate", "up", "down")) if mlp.get("shared") else None
-                y = routed_experts(h, w[p + "mlp.router"], ex, mlp["router"]["top"], sh)
+                y = routed_experts(h, w[p + "mlp.router"], ex, mlp["router"]["top"], sh, margins=route_margins)
             x = x + rms_norm(y, w[p + "norm2"], eps)
         if layers_out is not None:
             layers_out.append(x.clone())

@@ -35,12 +35,12 @@ def config(layers, vocab=90, width=40, taps=3, eps=1e-5, embed_scale=3.0):
 # latents wider than one lane pass, one tap (no history) and five
 CONFIGS = {
     "mixed": config([layer(), layer(mlp="moe"), layer(weights_of=0), layer(mlp="moe", top=1, shared_ff=0, experts=7, heads=2, window=9),
-                     layer(mlp=None, window=0), layer(mlp="moe", weights_of=1)]),
+                     layer(mlp=None, window=0, kv_rank=32, heads=8), layer(mlp="moe", weights_of=1)]),
     "odd": config([layer(heads=5, dim=6, rot_dim=6, rot_dims=4, vdim=10, q_rank=7, kv_rank=9, window=1, mlp="moe", experts=3, top=3,
                          expert_ff=5, shared_ff=7),
                    layer(heads=1, dim=3, rot_dim=2, vdim=5, q_rank=3, kv_rank=70, window=4, ff=17)],
                   vocab=75, width=36, taps=2, eps=1e-6, embed_scale=0.7),
-    "wide": config([layer(heads=9, dim=16, rot_dim=8, vdim=24, q_rank=48, kv_rank=136, window=70, ff=96),
+    "wide": config([layer(heads=9, dim=16, rot_dim=8, vdim=24, q_rank=48, kv_rank=144, window=70, ff=96),
                     layer(heads=2, dim=32, rot_dim=16, vdim=8, q_rank=24, kv_rank=264, window=0, mlp="moe", experts=70, top=4,
                           expert_ff=16, shared_ff=32)],
                    vocab=130, width=64, taps=5),

@@ -23,7 +23,7 @@ def test_config_reader_keeps_every_size_and_constant():
     assert (l1.ff_kind, l1.experts, l1.top, l1.expert_ff, l1.shared_ff) == ("moe", 5, 2, 12, 10)
     assert l2.weights_of == 0 and l5.weights_of == 1 and l1.weights_of is None
     assert (l3.experts, l3.top, l3.shared_ff, l3.mixer.heads, l3.mixer.window) == (7, 1, 0, 2, 9)
-    assert not l4.has_ff and l4.mixer.window == 0
+    assert not l4.has_ff and l4.mixer.window == 0 and l4.mixer.kv_rank == 32
     odd = fidizen.config_from_dict(CONFIGS["odd"])
     assert odd.layers[0].mixer.rot_dims == 4 and odd.layers[0].mixer.rot_dim == 6 and odd.norm_eps == 1e-6
     sh = fidizen.tensor_shapes(c)

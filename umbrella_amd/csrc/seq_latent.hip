@@ -305,15 +305,203 @@ extern "C" int umb_lat_attend(void* out, const float* qa, const UmbPagedKV* kv, 
   return UMB_OK;
 }
 
+// ---- prompt attention on the matrix pipe (16-bit storage; Dk a multiple of 8, kv_rank a multiple of 16).
+// Workgroup = (16 consecutive positions of one sequence, a block of 4 HPW heads); wave w owns HPW heads and walks the tile's
+// keys -- from the first position's window start to the last position -- in steps of 32, alone (no workgroup barrier).
+// Per step:  the 32 cached rows' first kv_rank features are copied to the wave's LDS tile (they are the VALUES, needed
+//            transposed below); the step is shared by the wave's HPW heads, which also share every key fragment load;
+//   S^T = K Q^T as two 16-key MFMA tiles per head (A = 16 keys x 32 features straight from the cached rows, B = the queries,
+//         rounded to the storage dtype once, when the tile starts);
+//   online softmax in fp32: lane (query j, key quad g) holds keys 4g .. 4g+3 of both tiles; the row maximum and sum are
+//         finished over the four lanes of a query by two shuffles; accumulators are rescaled when the maximum grows;
+//   O^T += V^T P^T: the lane's eight weights ARE its share of the B operand when V^T's k index runs over (tile 0: 4g .. 4g+3,
+//         tile 1: 4g .. 4g+3); V^T (A: 16 features x those 8 keys) is gathered from the LDS tile.
+// The sink joins the denominator at the end.  NSM / NVM bound the unrolled register arrays (key steps of 32 features, value
+// tiles of 16 features); the actual counts are run-time.
+template <typename P, int NSM, int NVM, int HPW>
+__global__ __launch_bounds__(256) void lat_attend_mfma_kernel(u16* __restrict__ out, const float* __restrict__ qa, UmbPagedKV kv,
+                                                              const u16* __restrict__ sink, const int* __restrict__ seq_slot,
+                                                              const int* __restrict__ seq_row0, const int* __restrict__ seq_pos0,
+                                                              const int* __restrict__ seq_len, int H, int Dc, int R, int window,
+                                                              float scale) {
+  extern __shared__ __attribute__((aligned(16))) u16 lat_lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g4 = lane >> 4;
+  const int Dk = Dc + R, LD = Dc + 8;                 // LDS row stride: 16 bytes of padding spread the key quads over the banks
+  const int ns = (Dk + 31) >> 5, nv = Dc >> 4;
+  u16* v_s = lat_lds + (long)wave * (32 * LD + 32 * 4);       // [32][LD] values, [32] 64-bit offsets
+  long* offs = reinterpret_cast<long*>(v_s + 32 * LD);
+  const int b = blockIdx.y;
+  const int n = seq_len[b], q0 = blockIdx.x * 16;
+  if (q0 >= n) return;
+  const int h0 = (blockIdx.z * 4 + wave) * HPW;
+  if (h0 >= H) return;
+  const int slot = seq_slot[b], row0 = seq_row0[b], pos0 = seq_pos0[b];
+  const int nq = n - q0 < 16 ? n - q0 : 16;
+  const int i_first = pos0 + q0, i_last = i_first + nq - 1;
+  const bool q_ok = j < nq;
+  const int i_j = i_first + (q_ok ? j : nq - 1);
+  const long qrow = row0 + q0 + (q_ok ? j : nq - 1);
+  const int j_lo = i_first - window + 1 > 0 ? i_first - window + 1 : 0;
+  const int total = i_last - j_lo + 1;
+  const u16* kbase = reinterpret_cast<const u16*>(kv.k);
+  u32x4 qf[HPW][NSM];
+  f32x4 o[HPW][NVM];
+  float m_run[HPW], l_run[HPW];
+  bool h_ok[HPW];
+#pragma unroll
+  for (int hh = 0; hh < HPW; ++hh) {
+    h_ok[hh] = h0 + hh < H;
+    const float* qr = qa + (qrow * H + (h_ok[hh] ? h0 + hh : h0)) * Dk;
+#pragma unroll
+    for (int s = 0; s < NSM; ++s) {
+      const int d = 32 * s + 8 * g4;
+      qf[hh][s] = u32x4{0u, 0u, 0u, 0u};
+      if (s < ns && d < Dk) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(qr + d), c = *reinterpret_cast<const f32x4*>(qr + d + 4);
+        qf[hh][s] = u32x4{pack2<P>(a[0], a[1]), pack2<P>(a[2], a[3]), pack2<P>(c[0], c[1]), pack2<P>(c[2], c[3])};
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < NVM; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run[hh] = -INFINITY;
+    l_run[hh] = 0.f;
+  }
+  const int pieces = 32 * (Dc >> 3);                 // 16-byte pieces of the step's value tile
+  for (int base = 0; base < total; base += 32) {
+    if (lane < 32) {
+      const int kx = base + lane;
+      offs[lane] = kx < total ? pkv_tok(kv, slot, j_lo + kx, 0, 1, Dk) : -1;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (int p = lane; p < pieces; p += 64) {
+      const int m = p / (Dc >> 3), dp = (p % (Dc >> 3)) * 8;
+      const long off = offs[m];
+      const u32x4 v = off >= 0 ? *reinterpret_cast<const u32x4*>(kbase + off + dp) : u32x4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(v_s + m * LD + dp) = v;
+    }
+    f32x4 sc[HPW][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int hh = 0; hh < HPW; ++hh) sc[hh][u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const long off = offs[16 * u + j];
+      const u16* kr = kbase + (off >= 0 ? off : 0);
+      u32x4 kf[NSM];
+#pragma unroll
+      for (int s = 0; s < NSM; ++s) {
+        const int d = 32 * s + 8 * g4;
+        kf[s] = (s < ns && d < Dk && off >= 0) ? *reinterpret_cast<const u32x4*>(kr + d) : u32x4{0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+      for (int s = 0; s < NSM; ++s) {
+        if (s < ns) {
+#pragma unroll
+          for (int hh = 0; hh < HPW; ++hh) sc[hh][u] = P::mfma(kf[s], qf[hh][s], sc[hh][u]);
+        }
+      }
+    }
+    u32x4 pf[HPW];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      float sv[8], mx = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int jt = j_lo + base + 16 * u + 4 * g4 + rr;
+          const bool vis = q_ok && jt <= i_j && jt > i_j - window;
+          sv[4 * u + rr] = vis ? sc[hh][u][rr] * scale : -INFINITY;
+          mx = fmaxf(mx, sv[4 * u + rr]);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[hh], mx);
+      const float fac = m_new == -INFINITY ? 1.f : expf(m_run[hh] - m_new);
+      float w[8], sum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        w[e] = sv[e] == -INFINITY ? 0.f : expf(sv[e] - m_new);
+        sum += w[e];
+      }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      l_run[hh] = l_run[hh] * fac + sum;
+      m_run[hh] = m_new;
+#pragma unroll
+      for (int dt = 0; dt < NVM; ++dt) {
+        if (dt < nv) { o[hh][dt][0] *= fac; o[hh][dt][1] *= fac; o[hh][dt][2] *= fac; o[hh][dt][3] *= fac; }
+      }
+      pf[hh] = u32x4{pack2<P>(w[0], w[1]), pack2<P>(w[2], w[3]), pack2<P>(w[4], w[5]), pack2<P>(w[6], w[7])};
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    // O^T[d][query] += V^T[d][keys] P^T[keys][query]: lane (d row j of tile dt, quad g4) gathers its 8 keys' values
+#pragma unroll
+    for (int dt = 0; dt < NVM; ++dt) {
+      if (dt < nv) {
+        unsigned e[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m) e[m] = v_s[((m >> 2) * 16 + 4 * g4 + (m & 3)) * LD + 16 * dt + j];
+        const u32x4 va = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) o[hh][dt] = P::mfma(va, pf[hh], o[hh][dt]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  // lane holds O^T[d = 16 dt + 4 g4 + rr][query j]
+  if (q_ok) {
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      if (!h_ok[hh]) continue;
+      const float sk = sink ? P::to_f(sink[h0 + hh]) : -INFINITY;
+      const float M = fmaxf(m_run[hh], sk);
+      const float f = expf(m_run[hh] - M);
+      const float inv = f / (l_run[hh] * f + (sink ? expf(sk - M) : 0.f));
+#pragma unroll
+      for (int dt = 0; dt < NVM; ++dt) {
+        if (dt < nv) {
+          u32x2 pk;
+          pk[0] = pack2<P>(o[hh][dt][0] * inv, o[hh][dt][1] * inv);
+          pk[1] = pack2<P>(o[hh][dt][2] * inv, o[hh][dt][3] * inv);
+          *reinterpret_cast<u32x2*>(out + (qrow * H + h0 + hh) * Dc + 16 * dt + 4 * g4) = pk;
+        }
+      }
+    }
+  }
+}
+
 extern "C" int umb_lat_attend_tiled_ok(int H, int kv_rank, int rot_dim, int dtype) {
-  (void)H; (void)kv_rank; (void)rot_dim; (void)dtype;
-  return 0;
+  const int Dk = kv_rank + rot_dim;
+  return H >= 1 && (dtype == UMB_SEQ_BF16 || dtype == UMB_SEQ_F16) && kv_rank >= 16 && kv_rank % 16 == 0 && kv_rank <= 512 &&
+         rot_dim >= 0 && Dk % 8 == 0 && Dk <= 576;
 }
 
 extern "C" int umb_lat_attend_tiled(void* out, const float* qa, const UmbPagedKV* kv, const void* sink, const int* seq_slot,
                                     const int* seq_row0, const int* seq_pos0, const int* seq_len, int B, int max_len, int H,
                                     int kv_rank, int rot_dim, int window, float scale, int dtype, hipStream_t st) {
-  (void)out; (void)qa; (void)kv; (void)sink; (void)seq_slot; (void)seq_row0; (void)seq_pos0; (void)seq_len; (void)B;
-  (void)max_len; (void)H; (void)kv_rank; (void)rot_dim; (void)window; (void)scale; (void)dtype; (void)st;
-  return UMB_EINVAL;
+  if (B < 1 || max_len < 1 || window < 1 || !out || !qa || !lat_kv_ok(kv) || !seq_slot || !seq_row0 || !seq_pos0 || !seq_len ||
+      !umb_lat_attend_tiled_ok(H, kv_rank, rot_dim, dtype))
+    return UMB_EINVAL;
+  const int Dk = kv_rank + rot_dim;
+  const size_t lds = 4 * (size_t)(32 * (kv_rank + 8) + 128) * sizeof(u16);
+#define LAT_MFMA(NSM, NVM, HPW)                                                                                            \
+  do {                                                                                                                     \
+    const dim3 grid((max_len + 15) / 16, B, (H + 4 * HPW - 1) / (4 * HPW));                                                \
+    if (ensure_dynamic_lds<lat_attend_mfma_kernel<P, NSM, NVM, HPW>>(lds) != UMB_OK) return UMB_EHIP;                      \
+    hipLaunchKernelGGL((lat_attend_mfma_kernel<P, NSM, NVM, HPW>), grid, dim3(256), lds, st, (u16*)out, qa, *kv,           \
+                       (const u16*)sink, seq_slot, seq_row0, seq_pos0, seq_len, H, kv_rank, rot_dim, window, scale);       \
+  } while (0)
+#define LAT_MFMA_SHAPE()                                                                                                   \
+  if (Dk <= 128 && kv_rank <= 128) { if (H >= 8) LAT_MFMA(4, 8, 2); else LAT_MFMA(4, 8, 1); }                              \
+  else if (Dk <= 320 && kv_rank <= 256) { if (H >= 8) LAT_MFMA(10, 16, 2); else LAT_MFMA(10, 16, 1); }                     \
+  else LAT_MFMA(18, 32, 1)
+  if (dtype == UMB_SEQ_BF16) { using P = BF16; LAT_MFMA_SHAPE(); }
+  else { using P = F16; LAT_MFMA_SHAPE(); }
+#undef LAT_MFMA_SHAPE
+#undef LAT_MFMA
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
 }
