@@ -48,10 +48,11 @@ int umb_seq_linear(void* out, const void* x, const void* w, const void* bias, in
 int umb_seq_linear_batched(void* out, const void* x, const void* w, int T, int N, int K, int ldx, int ldo, int batch, long sx,
                            long sw, long so, int epi, const float* gate, int ldg, int sg, int dtype, umb_stream_t stream);
 /* Grouped product over row ranges read from device memory: tile i (blockIdx.y, i < max_tiles) is {group, first row, rows}
- * (3 int32, rows <= 64, rows == 0: nothing); its rows of x [*][K] meet w + group * gs ([N][K], or the stacked [2N'][K] of
- * epi 2) and land in the same rows of out.  No bias. */
-int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, long gs, int N, int K,
-                           int epi, int dtype, umb_stream_t stream);
+ * (3 int32, rows <= tile_rows, rows == 0: nothing); its rows of x [*][K] meet w + group * gs ([N][K], or the stacked
+ * [2N'][K] of epi 2) and land in the same rows of out.  No bias.  tile_rows 64: weights streamed per tile (few rows per
+ * group); 128: both operands staged through LDS (16-bit storage, K and gs multiples of 8). */
+int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows, long gs,
+                           int N, int K, int epi, int dtype, umb_stream_t stream);
 
 /* RMS norm in `groups` equal consecutive parts of a row: part / sqrt(mean(part^2) + eps), whole row times w.
  * x fp32 [*][W]; rows: optional gather (row i of out comes from row rows[i] of x); out_f32 and/or out_dt may be given. */
@@ -81,6 +82,12 @@ int umb_canon_update(float* state, const float* x, const int* seq_slot, const in
 int umb_canon_step(void* h, const float* x, const void* w, float* state, const int* pos, const int* slot, int T, int W,
                    int taps, int dtype, umb_stream_t stream);
 
+/* The seam x <- x + group_norm(y) * w_post followed by that convolution, for steps of one token per sequence, in one
+ * launch: h = canon(x), the state row of the token's position is overwritten with the new x.  W / groups <= 8192. */
+int umb_seq_resid_canon_step(float* x, void* h, const float* y, const void* w_post, const void* canon, float* state,
+                             const int* pos, const int* slot, int T, int W, int groups, int taps, float eps, int dtype,
+                             umb_stream_t stream);
+
 /* ---- PolyNorm activation: out[t] = a N(z) + b N(z^2) + c N(z^3) + e with powers element by element and
  * N(v) = v / sqrt(mean(v^2) + eps) over the row; coef = {a, b, c, e} in `dtype`; z fp32 [T][F], out in `dtype`. */
 int umb_polynorm(void* out, const float* z, const void* coef, int T, int F, float eps, int dtype, umb_stream_t stream);
@@ -90,9 +97,10 @@ int umb_polynorm(void* out, const float* z, const void* coef, int T, int F, floa
  * itself.  sel [T][top] expert ids, wt [T][top] fp32. */
 int umb_moe_route(int* sel, float* wt, const float* logits, int T, int E, int top, umb_stream_t stream);
 /* orders the T*top (token, choice) pairs by expert: pos_of [T*top] = row of the pair in the expert-ordered list,
- * tiles [max_tiles][3] = {expert, first row, rows} covering every expert's rows in pieces of at most 64
- * (max_tiles >= ceil(T top / 64) + E; unused entries get rows = 0). */
-int umb_moe_plan(int* pos_of, int* tiles, const int* sel, int T, int E, int top, int max_tiles, umb_stream_t stream);
+ * tiles [max_tiles][3] = {expert, first row, rows} covering every expert's rows in pieces of at most tile_rows
+ * (max_tiles >= ceil(T top / tile_rows) + E; unused entries get rows = 0). */
+int umb_moe_plan(int* pos_of, int* tiles, const int* sel, int T, int E, int top, int max_tiles, int tile_rows,
+                 umb_stream_t stream);
 /* xs[pos_of[t top + k]] = wt[t][k] * h[t]  (the weight multiplies the expert's INPUT); h, xs in `dtype` */
 int umb_moe_scatter(void* xs, const void* h, const float* wt, const int* pos_of, int T, int W, int top, int dtype,
                     umb_stream_t stream);

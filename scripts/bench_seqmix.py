@@ -1,7 +1,12 @@
-"""Prefill and decode throughput of the sequence-mixer family (Gitopel) at layer sizes that resemble real models, beside the
-framework's Llama runtime at equal width / feed-forward / head sizes and layer count.  Random weights, synthetic ids.
+"""Prefill and decode throughput of the sequence-mixer family at layer sizes that resemble real models.  Random weights,
+synthetic ids.
 
     python bench.py --family gitopel [--sizes 1b,8b] [--prompt-len 2048] [--decode-steps 64] [--batch 16]
+        Gitopel beside the framework's Llama runtime at equal width / feed-forward / head sizes and layer count
+    python bench.py --family fidizen [--sizes 1b,8b] ...
+        Fidizen (latent attention, dense PolyNorm and routed-expert feed-forwards) beside Gitopel's windowed-attention
+        layers -- the closest existing model: same runtime, cache manager and engine -- at equal width, heads, window,
+        feed-forward width and layer count
 
 or directly: python scripts/bench_seqmix.py.  One JSON line: per size, ms and tokens/s of
   prefill   one prompt of --prompt-len tokens in one step (Llama: its chunked prompt path)
@@ -30,6 +35,32 @@ SIZES = {
 }
 
 
+# Fidizen: per head `dim` unrotated + `rot` rotated features, value size vdim, latents q_rank / kv_rank; layers alternate a
+# dense feed-forward (width ff) and experts (each ff / 4 wide, two of eight used, plus a shared one: ff / 2 active per token)
+FID_SIZES = {
+    "1b": dict(width=2048, ff=8192, heads=16, dim=64, rot=32, vdim=64, q_rank=768, kv_rank=256, window=512, experts=8, top=2,
+               layers=4, vocab=32000),
+    "8b": dict(width=4096, ff=14336, heads=32, dim=128, rot=64, vdim=128, q_rank=1536, kv_rank=512, window=1024, experts=8,
+               top=2, layers=2, vocab=32000),
+}
+
+
+def fidizen_config(s):
+    mixer = {"heads": s["heads"], "dim": s["dim"], "rot_dim": s["rot"], "vdim": s["vdim"], "q_rank": s["q_rank"],
+             "kv_rank": s["kv_rank"], "mask": {"size": s["window"]}, "rot": {"dims": s["rot"], "base": 10000.0},
+             "scale": (s["dim"] + s["rot"]) ** -0.5}
+    layers = []
+    for i in range(s["layers"]):
+        if i % 2 == 0:
+            mlp = {"kind": "dense", "ff": s["ff"]}
+        else:
+            mlp = {"kind": "moe", "router": {"experts": s["experts"], "top": s["top"]}, "expert": {"ff": s["ff"] // 4},
+                   "shared": {"ff": s["ff"] // 4}}
+        layers.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Fidizen", "layers": layers, "norm": {"eps": 1e-6}, "canon": {"taps": 4},
+            "embedding": {"scale": s["width"] ** 0.5}, "vocab": s["vocab"], "width": s["width"]}
+
+
 def gitopel_config(s):
     layers = []
     for ch in s["pattern"]:
@@ -44,12 +75,12 @@ def gitopel_config(s):
     return {"architecture": "Gitopel", "layers": layers, "norm": {"eps": 1e-6, "groups": 4}, "vocab": s["vocab"], "width": s["width"]}
 
 
-def device_state(cfg, dtype, seed=0, rank=16):
+def device_state(cfg, dtype, seed=0, rank=16, shapes=None):
     """random checkpoint drawn on the device in the storage dtype"""
     from umbrella_amd.models import gitopel
     g = torch.Generator(device="cuda").manual_seed(seed)
     sd = {}
-    for name, shape in gitopel.tensor_shapes(cfg, rank).items():
+    for name, shape in (shapes or gitopel.tensor_shapes(cfg, rank)).items():
         leaf = name.split(".")[-1]
         if "norm" in leaf:
             sd[name] = torch.ones(shape, dtype=dtype, device="cuda")
@@ -69,12 +100,18 @@ def timed(fn, reps):
     return (time.time() - t0) / reps * 1e3
 
 
-def bench_gitopel(s, args, dtype):
+def bench_gitopel(s, args, dtype, fidizen=False):
+    from umbrella_amd.models import fidizen as fid
     from umbrella_amd.models import gitopel
-    cfg = gitopel.config_from_dict(gitopel_config(s))
     B, P, steps = args.batch, args.prompt_len, args.decode_steps
-    m = gitopel.Gitopel("bench", batch_size=B + 1, max_length=P + 2 * steps + 8, max_tokens=(B + 1) * (P + 2 * steps + 8),
-                        device="cuda:0", dtype=dtype, state_dict=device_state(cfg, dtype), config=cfg, max_step_tokens=max(P, B))
+    kw = dict(batch_size=B + 1, max_length=P + 2 * steps + 8, max_tokens=(B + 1) * (P + 2 * steps + 8), device="cuda:0",
+              dtype=dtype, max_step_tokens=max(P, B))
+    if fidizen:
+        cfg = fid.config_from_dict(fidizen_config(s))
+        m = fid.Fidizen("bench", state_dict=device_state(cfg, dtype, shapes=fid.tensor_shapes(cfg)), config=cfg, **kw)
+    else:
+        cfg = gitopel.config_from_dict(gitopel_config(s))
+        m = gitopel.Gitopel("bench", state_dict=device_state(cfg, dtype), config=cfg, **kw)
     m.alloc()
     ids = torch.randint(0, s["vocab"], (P,), generator=torch.Generator().manual_seed(1)).tolist()
     out = {"weight_GB": round(m.weight_bytes() / 1e9, 3)}
@@ -130,6 +167,31 @@ def bench_llama(s, args, dtype):
     return out
 
 
+def run_fidizen(args):
+    """Fidizen beside Gitopel's windowed-attention layers at equal width, heads x head size, window, feed-forward width and
+    layer count"""
+    import __graft_entry__ as ge
+    ge.build_seq()
+    dtype = torch.bfloat16
+    res = {}
+    for name in args.sizes.split(","):
+        s = FID_SIZES[name]
+        res[name] = {"shape": dict(s)}
+        res[name]["fidizen"] = bench_gitopel(s, args, dtype, fidizen=True)
+        torch.cuda.empty_cache()
+        if not args.no_gitopel:
+            hd = s["dim"] + s["rot"]
+            g = dict(width=s["width"], ff=s["ff"], heads=s["heads"], kv_heads=max(1, s["heads"] // 4), dim=hd, window=s["window"],
+                     pool=16, pattern="a" * s["layers"], vocab=s["vocab"])
+            res[name]["gitopel_attention_equal_size"] = bench_gitopel(g, args, dtype)
+            torch.cuda.empty_cache()
+    line = {"metric": "prefill / decode throughput, Fidizen beside Gitopel's attention layers at equal size", "unit": "tokens/s",
+            "dtype": "bf16", "data": "synthetic: random weights, random ids", "n_gpus": 1, "prompt_len": args.prompt_len,
+            "decode_steps": args.decode_steps, "batch": args.batch, "sizes": res}
+    print(json.dumps(line), flush=True)
+    return line
+
+
 def run(args):
     import __graft_entry__ as ge
     ge.build()
@@ -162,5 +224,7 @@ def add_args(ap):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--family", default="gitopel", choices=["gitopel", "fidizen"])
     add_args(ap)
-    run(ap.parse_args())
+    a = ap.parse_args()
+    run_fidizen(a) if a.family == "fidizen" else run(a)

@@ -253,14 +253,15 @@ _PKV = C.POINTER(UmbPagedKV)
 SEQ_SIGNATURES = {
     "umb_seq_linear": [_P, _P, _P, _P, _I, _I, _I, _I, _I],
     "umb_seq_linear_batched": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _L, _I, _P, _I, _I, _I],
-    "umb_seq_linear_grouped": [_P, _P, _P, _P, _I, _L, _I, _I, _I, _I],
+    "umb_seq_linear_grouped": [_P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I],
     "umb_seq_embed": [_P, _P, _P, _F, _I, _I, _I, _I],
     "umb_canon_conv": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I],
     "umb_canon_update": [_P, _P, _P, _P, _P, _P, _I, _I, _I],
     "umb_canon_step": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I],
+    "umb_seq_resid_canon_step": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I],
     "umb_polynorm": [_P, _P, _P, _I, _I, _F, _I],
     "umb_moe_route": [_P, _P, _P, _I, _I, _I],
-    "umb_moe_plan": [_P, _P, _P, _I, _I, _I, _I],
+    "umb_moe_plan": [_P, _P, _P, _I, _I, _I, _I, _I],
     "umb_moe_scatter": [_P, _P, _P, _P, _I, _I, _I, _I],
     "umb_moe_combine": [_P, _P, _P, _I, _I, _I, _I],
     "umb_lat_prep": [_P, _PKV, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I],

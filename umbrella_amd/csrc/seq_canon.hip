@@ -22,27 +22,27 @@ __global__ __launch_bounds__(256) void embed_kernel(float* __restrict__ x, const
   for (int i = threadIdx.x; i < W; i += 256) x[(long)t * W + i] = ldf<P>(embed + (long)tok * W + i) * scale;
 }
 
-// FUSED: T == number of sequences, one token each; the state row of the token's own position is written after the reads
+// FUSED: T == number of sequences, one token each; the state row of the token's own position is written after the reads.
+// One thread per (token, channel); the loads of the taps do not depend on one another.
 template <typename P, bool FUSED>
 __global__ __launch_bounds__(256) void canon_conv_kernel(typename El<P>::type* __restrict__ h, const float* __restrict__ x,
                                                          const typename El<P>::type* __restrict__ w, float* __restrict__ state,
                                                          const int* __restrict__ pos, const int* __restrict__ slot, int W,
                                                          int taps) {
-  const int t = blockIdx.x, p = pos[t], sl = slot[t];
-  const int S = taps - 1;
-  for (int c = threadIdx.x; c < W; c += 256) {
-    const float own = x[(long)t * W + c];
-    float a = own * (1.f + ldf<P>(w + (long)c * taps + S));
-    for (int k = 1; k <= S; ++k) {
-      if (p - k < 0) break;
-      float v;
-      if (!FUSED && t - k >= 0 && slot[t - k] == sl) v = x[(long)(t - k) * W + c];
-      else v = state[((long)sl * S + (p - k) % S) * W + c];
-      a += ldf<P>(w + (long)c * taps + S - k) * v;
-    }
-    stf<P>(h + (long)t * W + c, a);
-    if (FUSED && S > 0) state[((long)sl * S + p % S) * W + c] = own;
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= W) return;
+  const int p = pos[t], sl = slot[t], S = taps - 1;
+  const float own = x[(long)t * W + c];
+  float a = own * (1.f + ldf<P>(w + (long)c * taps + S));
+  for (int k = 1; k <= S; ++k) {
+    const bool in = p - k >= 0;
+    const bool here = !FUSED && t - k >= 0 && slot[t - k < 0 ? 0 : t - k] == sl;
+    const float* src = here ? x + (long)(t - k) * W + c : state + ((long)sl * S + (in ? p - k : 0) % S) * W + c;
+    const float v = *src;
+    a += in ? ldf<P>(w + (long)c * taps + S - k) * v : 0.f;
   }
+  stf<P>(h + (long)t * W + c, a);
+  if (FUSED && S > 0) state[((long)sl * S + p % S) * W + c] = own;
 }
 
 __global__ __launch_bounds__(256) void canon_update_kernel(float* __restrict__ state, const float* __restrict__ x,
@@ -74,7 +74,7 @@ extern "C" int umb_canon_conv(void* h, const float* x, const void* w, const floa
   if (T < 1 || W < 1 || taps < 1 || !h || !x || !w || !pos || !slot || (taps > 1 && !state)) return UMB_EINVAL;
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
-    hipLaunchKernelGGL((canon_conv_kernel<P, false>), dim3(T), dim3(256), 0, st, (E*)h, x, (const E*)w, const_cast<float*>(state),
+    hipLaunchKernelGGL((canon_conv_kernel<P, false>), dim3(T, (W + 255) / 256), dim3(256), 0, st, (E*)h, x, (const E*)w, const_cast<float*>(state),
                        pos, slot, W, taps);
   })
   UMB_LAUNCH_CHECK();
@@ -97,7 +97,7 @@ extern "C" int umb_canon_step(void* h, const float* x, const void* w, float* sta
   if (T < 1 || W < 1 || taps < 1 || !h || !x || !w || !pos || !slot || (taps > 1 && !state)) return UMB_EINVAL;
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
-    hipLaunchKernelGGL((canon_conv_kernel<P, true>), dim3(T), dim3(256), 0, st, (E*)h, x, (const E*)w, state, pos, slot, W, taps);
+    hipLaunchKernelGGL((canon_conv_kernel<P, true>), dim3(T, (W + 255) / 256), dim3(256), 0, st, (E*)h, x, (const E*)w, state, pos, slot, W, taps);
   })
   UMB_LAUNCH_CHECK();
   return UMB_OK;

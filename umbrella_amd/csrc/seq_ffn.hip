@@ -20,9 +20,19 @@ __global__ __launch_bounds__(256) void polynorm_kernel(typename El<P>::type* __r
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float* zr = z + (long)t * F;
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-  for (int i = threadIdx.x; i < F; i += 256) {
-    const float v = zr[i], v2 = v * v;
-    s2 += v2; s4 += v2 * v2; s6 += v2 * v2 * v2;
+  const bool vec = (F & 3) == 0;
+  if (vec) {                                     // 16-byte loads, four in flight per thread
+#pragma unroll 4
+    for (int i = 4 * threadIdx.x; i < F; i += 1024) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(zr + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { const float v2 = v[e] * v[e]; s2 += v2; s4 += v2 * v2; s6 += v2 * v2 * v2; }
+    }
+  } else {
+    for (int i = threadIdx.x; i < F; i += 256) {
+      const float v = zr[i], v2 = v * v;
+      s2 += v2; s4 += v2 * v2; s6 += v2 * v2 * v2;
+    }
   }
   s2 = wave_sum(s2); s4 = wave_sum(s4); s6 = wave_sum(s6);
   if (lane == 0) { red[0][wave] = s2; red[1][wave] = s4; red[2][wave] = s6; }
@@ -32,9 +42,18 @@ __global__ __launch_bounds__(256) void polynorm_kernel(typename El<P>::type* __r
   s6 = red[2][0] + red[2][1] + red[2][2] + red[2][3];
   const float a = ldf<P>(coef) / sqrtf(s2 / (float)F + eps), b = ldf<P>(coef + 1) / sqrtf(s4 / (float)F + eps),
               c = ldf<P>(coef + 2) / sqrtf(s6 / (float)F + eps), e = ldf<P>(coef + 3);
-  for (int i = threadIdx.x; i < F; i += 256) {
-    const float v = zr[i];
-    stf<P>(out + (long)t * F + i, a * v + b * (v * v) + c * (v * v * v) + e);
+  if (vec) {
+#pragma unroll 4
+    for (int i = 4 * threadIdx.x; i < F; i += 1024) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(zr + i);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) stf<P>(out + (long)t * F + i + k, a * v[k] + b * (v[k] * v[k]) + c * (v[k] * v[k] * v[k]) + e);
+    }
+  } else {
+    for (int i = threadIdx.x; i < F; i += 256) {
+      const float v = zr[i];
+      stf<P>(out + (long)t * F + i, a * v + b * (v * v) + c * (v * v * v) + e);
+    }
   }
 }
 
@@ -72,7 +91,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int* __restrict__ sel, f
 
 // single workgroup: counts per expert (LDS atomics), row offsets, tile list, then every pair's row
 __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ pos_of, int* __restrict__ tiles,
-                                                        const int* __restrict__ sel, int pairs, int E, int max_tiles) {
+                                                        const int* __restrict__ sel, int pairs, int E, int max_tiles, int TR) {
   extern __shared__ int sm[];                 // [E] counts, [E] offsets / cursors
   int* cnt = sm;
   int* cur = sm + E;
@@ -84,8 +103,8 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ pos_of
     int off = 0, nt = 0;
     for (int e = 0; e < E; ++e) {
       cur[e] = off;
-      for (int r = 0; r < cnt[e]; r += 64) {
-        if (nt < max_tiles) { tiles[3 * nt] = e; tiles[3 * nt + 1] = off + r; tiles[3 * nt + 2] = cnt[e] - r < 64 ? cnt[e] - r : 64; }
+      for (int r = 0; r < cnt[e]; r += TR) {
+        if (nt < max_tiles) { tiles[3 * nt] = e; tiles[3 * nt + 1] = off + r; tiles[3 * nt + 2] = cnt[e] - r < TR ? cnt[e] - r : TR; }
         ++nt;
       }
       off += cnt[e];
@@ -133,11 +152,14 @@ extern "C" int umb_moe_route(int* sel, float* wt, const float* logits, int T, in
   return UMB_OK;
 }
 
-extern "C" int umb_moe_plan(int* pos_of, int* tiles, const int* sel, int T, int E, int top, int max_tiles, hipStream_t st) {
+extern "C" int umb_moe_plan(int* pos_of, int* tiles, const int* sel, int T, int E, int top, int max_tiles, int tile_rows,
+                            hipStream_t st) {
   const long pairs = (long)T * top;
-  if (T < 1 || E < 1 || E > 4096 || top < 1 || pairs > 0x7fffffffL || max_tiles < (pairs + 63) / 64 + E || !pos_of || !tiles || !sel)
+  if (T < 1 || E < 1 || E > 4096 || top < 1 || pairs > 0x7fffffffL || tile_rows < 1 ||
+      max_tiles < (pairs + tile_rows - 1) / tile_rows + E || !pos_of || !tiles || !sel)
     return UMB_EINVAL;
-  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 2 * E * sizeof(int), st, pos_of, tiles, sel, (int)pairs, E, max_tiles);
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 2 * E * sizeof(int), st, pos_of, tiles, sel, (int)pairs, E, max_tiles,
+                     tile_rows);
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }

@@ -205,11 +205,22 @@ __global__ __launch_bounds__(256) void seq_linear_kernel(void* __restrict__ out_
 template <typename P, bool DUAL>
 __global__ __launch_bounds__(256) void seq_linear_wide_kernel(void* __restrict__ out_, const u16* __restrict__ x,
                                                               const u16* __restrict__ w, const u16* __restrict__ bias, int T,
-                                                              int N, int K, int epi) {
+                                                              int N, int K, int epi, LinExt ext) {
   __shared__ __attribute__((aligned(16))) u16 tile[2][2][2][128 * 32];      // [buffer][A | B][k half][row][32 k]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, g = lane >> 4;
   const int wm = wave >> 1, wn = wave & 1;
-  const int n0 = blockIdx.x * (DUAL ? 64 : 128), t0 = blockIdx.y * 128;
+  int t0 = blockIdx.y * 128;
+  long obase = 0;
+  if (ext.tiles) {                         // grouped: a tile of up to 128 rows of one group
+    const int* td = ext.tiles + 3 * blockIdx.y;
+    if (td[2] <= 0) return;
+    w += (long)td[0] * ext.gs;
+    x += (long)td[1] * K;
+    obase = (long)td[1] * N;
+    T = td[2];
+    t0 = 0;
+  }
+  const int n0 = blockIdx.x * (DUAL ? 64 : 128);
   // staging: thread owns chunks c = tid + 256 i (i < 4) of each operand's 128 x 8 chunk grid: row c / 8, 16-byte chunk c % 8
   const u16* asrc[4];
   const u16* bsrc[4];
@@ -287,11 +298,11 @@ __global__ __launch_bounds__(256) void seq_linear_wide_kernel(void* __restrict__
         float sv = acc[i][tt][r] + (bias ? P::to_f(bias[n]) : 0.f);
         if constexpr (DUAL) {
           const float uv = acc[i + 2][tt][r] + (bias ? P::to_f(bias[N + n]) : 0.f);
-          reinterpret_cast<u16*>(out_)[(long)t * N + n] = P::from_f(siluf_(sv) * uv);
+          reinterpret_cast<u16*>(out_)[obase + (long)t * N + n] = P::from_f(siluf_(sv) * uv);
         } else if (epi == EPI_DT) {
-          reinterpret_cast<u16*>(out_)[(long)t * N + n] = P::from_f(sv);
+          reinterpret_cast<u16*>(out_)[obase + (long)t * N + n] = P::from_f(sv);
         } else {
-          reinterpret_cast<float*>(out_)[(long)t * N + n] = sv;
+          reinterpret_cast<float*>(out_)[obase + (long)t * N + n] = sv;
         }
       }
     }
@@ -299,14 +310,16 @@ __global__ __launch_bounds__(256) void seq_linear_wide_kernel(void* __restrict__
 }
 
 template <typename P>
-static int launch_wide(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st) {
+static int launch_wide(void* out, const void* x, const void* w, const void* bias, int T, int N, int K, int epi, hipStream_t st,
+                       const LinExt& ext = LinExt{0, 0, 0, 0, 0, 0, nullptr, nullptr, 0, 0}, int gy = 0) {
   if constexpr (sizeof(typename El<P>::type) == 2) {
+    const unsigned ty = gy > 0 ? gy : (T + 127) / 128;
     if (epi == EPI_SILU_MUL)
-      hipLaunchKernelGGL((seq_linear_wide_kernel<P, true>), dim3((N + 63) / 64, (T + 127) / 128), dim3(256), 0, st, out,
-                         (const u16*)x, (const u16*)w, (const u16*)bias, T, N, K, epi);
+      hipLaunchKernelGGL((seq_linear_wide_kernel<P, true>), dim3((N + 63) / 64, ty), dim3(256), 0, st, out,
+                         (const u16*)x, (const u16*)w, (const u16*)bias, T, N, K, epi, ext);
     else
-      hipLaunchKernelGGL((seq_linear_wide_kernel<P, false>), dim3((N + 127) / 128, (T + 127) / 128), dim3(256), 0, st, out,
-                         (const u16*)x, (const u16*)w, (const u16*)bias, T, N, K, epi);
+      hipLaunchKernelGGL((seq_linear_wide_kernel<P, false>), dim3((N + 127) / 128, ty), dim3(256), 0, st, out,
+                         (const u16*)x, (const u16*)w, (const u16*)bias, T, N, K, epi, ext);
     UMB_LAUNCH_CHECK();
     return UMB_OK;
   } else {
@@ -375,14 +388,21 @@ extern "C" int umb_seq_linear_batched(void* out, const void* x, const void* w, i
   })
 }
 
-extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, long gs, int N,
-                                      int K, int epi, int dtype, hipStream_t st) {
-  if (max_tiles < 1 || max_tiles > 65535 || N < 1 || K < 1 || epi < 0 || epi > 2 || !out || !x || !w || !tiles) return UMB_EINVAL;
+extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows,
+                                      long gs, int N, int K, int epi, int dtype, hipStream_t st) {
+  if (max_tiles < 1 || max_tiles > 65535 || N < 1 || K < 1 || epi < 0 || epi > 2 || !out || !x || !w || !tiles ||
+      (tile_rows != 64 && tile_rows != 128))
+    return UMB_EINVAL;
   if (epi == EPI_SILU_MUL) {
     if (N & 1) return UMB_EINVAL;
     N >>= 1;
   }
   const LinExt ext{K, N, 0, 0, 0, gs, tiles, nullptr, 0, 0};
+  if (tile_rows == 128) {                  // many rows per group: both operands staged through LDS (16-bit storage only)
+    if (dtype == UMB_SEQ_F32 || K % 8 || gs % 8) return UMB_EINVAL;
+    if (dtype == UMB_SEQ_BF16) return launch_wide<BF16>(out, x, w, nullptr, 128, N, K, epi, st, ext, max_tiles);
+    return launch_wide<F16>(out, x, w, nullptr, 128, N, K, epi, st, ext, max_tiles);
+  }
   DISPATCH_SEQ_DTYPE(dtype, {
     if (K % 8 == 0 && gs % 8 == 0) {
       if (N >= 64 && sizeof(typename El<P>::type) == 2) return launch_tt<P, 4, 4, true>(out, x, w, nullptr, 64, N, K, epi, st, ext, max_tiles);

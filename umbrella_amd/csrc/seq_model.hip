@@ -24,13 +24,29 @@ static const void* first_norm_of(const UmbSeqModel* m, int l) { return l < m->L 
 // What a sublayer reads.  With a pre-norm the seam kernel has already left norm(x) * w in ws->h.  Without one the sublayer
 // reads the residual stream itself through the causal convolution x + conv(x), whose last inputs are the sequence's state.
 static int sublayer_input(const UmbSeqModel* m, const UmbSeqWork* ws, const UmbSeqStep* s, const void* pre_norm, const void* canon,
-                          float* canon_state, hipStream_t st) {
+                          float* canon_state, bool h_ready, hipStream_t st) {
   const int T = s->T, W = m->W, dt = m->dtype;
   if (pre_norm) return canon ? UMB_EINVAL : UMB_OK;           // a convolution on normed inputs is not implemented
+  if (h_ready) return UMB_OK;                                 // the seam before it has already run the convolution
   if (!canon) return UMB_EINVAL;                              // every design so far has one of the two
   if (s->max_len == 1) return umb_canon_step(ws->h, ws->x, canon, canon_state, s->pos, s->slot, T, W, m->canon_taps, dt, st);
   SEQ_TRY(umb_canon_conv(ws->h, ws->x, canon, canon_state, s->pos, s->slot, T, W, m->canon_taps, dt, st));
   return umb_canon_update(canon_state, ws->x, s->seq_slot, s->seq_row0, s->seq_pos0, s->seq_len, s->B, W, m->canon_taps, st);
+}
+
+// The seam behind a sublayer: x <- x + norm(y) * w_post, and what the NEXT sublayer reads.  With a pre-norm that is
+// norm(x) * w_next (same kernel).  Without one, a step of one token per sequence also runs the next sublayer's convolution
+// and state update here (*h_ready); longer steps leave it to sublayer_input, where a token's neighbours are complete.
+static int seam(const UmbSeqModel* m, const UmbSeqWork* ws, const UmbSeqStep* s, const void* w_post, const void* w_next,
+                const void* next_canon, float* next_state, bool* h_ready, hipStream_t st) {
+  const int T = s->T, W = m->W;
+  *h_ready = false;
+  if (!w_next && next_canon && s->max_len == 1 && W / m->groups <= 8192) {
+    *h_ready = true;
+    return umb_seq_resid_canon_step(ws->x, ws->h, ws->y, w_post, next_canon, next_state, s->pos, s->slot, T, W, m->groups,
+                                    m->canon_taps, m->eps, m->dtype, st);
+  }
+  return umb_seq_resid_norm(ws->x, ws->h, ws->y, w_post, w_next, T, W, m->groups, m->eps, m->dtype, st);
 }
 
 // feed-forward of ws->h into ws->y (fp32)
@@ -52,7 +68,9 @@ static int feed_forward(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSe
         !ws->moe_tiles || !ws->moe_xs || !ws->moe_act || !ws->moe_y || ly.router.N != E)
       return UMB_EINVAL;
     const long pairs = (long)T * top;
-    const int max_tiles = (int)((pairs + 63) / 64) + E;
+    // many rows per expert (prompts): tiles of 128 rows on the LDS-staged kernel; few (decoding): tiles of 64, weights streamed
+    const int tr = (dt != UMB_SEQ_F32 && pairs >= 64L * E && W % 8 == 0 && F % 8 == 0) ? 128 : 64;
+    const int max_tiles = (int)((pairs + tr - 1) / tr) + E;
     if (max_tiles > ws->moe_max_tiles) return UMB_EINVAL;
     if (ly.s_gu.w) {                                                           // the shared expert sees every token
       SEQ_TRY(lin(ly.s_gu, ws->act, ws->h, T, 2, dt, st));
@@ -60,10 +78,10 @@ static int feed_forward(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSe
     }
     SEQ_TRY(lin(ly.router, ws->proj, ws->h, T, 0, dt, st));
     SEQ_TRY(umb_moe_route(ws->moe_sel, ws->moe_wt, ws->proj, T, E, top, st));
-    SEQ_TRY(umb_moe_plan(ws->moe_pos, ws->moe_tiles, ws->moe_sel, T, E, top, max_tiles, st));
+    SEQ_TRY(umb_moe_plan(ws->moe_pos, ws->moe_tiles, ws->moe_sel, T, E, top, max_tiles, tr, st));
     SEQ_TRY(umb_moe_scatter(ws->moe_xs, ws->h, ws->moe_wt, ws->moe_pos, T, W, top, dt, st));
-    SEQ_TRY(umb_seq_linear_grouped(ws->moe_act, ws->moe_xs, ly.e_gu, ws->moe_tiles, max_tiles, 2L * F * W, 2 * F, W, 2, dt, st));
-    SEQ_TRY(umb_seq_linear_grouped(ws->moe_y, ws->moe_act, ly.e_down, ws->moe_tiles, max_tiles, (long)W * F, W, F, 0, dt, st));
+    SEQ_TRY(umb_seq_linear_grouped(ws->moe_act, ws->moe_xs, ly.e_gu, ws->moe_tiles, max_tiles, tr, 2L * F * W, 2 * F, W, 2, dt, st));
+    SEQ_TRY(umb_seq_linear_grouped(ws->moe_y, ws->moe_act, ly.e_down, ws->moe_tiles, max_tiles, tr, (long)W * F, W, F, 0, dt, st));
     return umb_moe_combine(ws->y, ws->moe_y, ws->moe_pos, T, W, top, ly.s_gu.w ? 1 : 0, st);
   }
   return UMB_EINVAL;
@@ -78,10 +96,12 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
     SEQ_TRY(umb_seq_embed_norm(ws->x, ws->h, m->embed, s->tokens, m->layers[0].norm1, T, W, m->V, groups, eps, dt, st));
   else
     SEQ_TRY(umb_seq_embed(ws->x, m->embed, s->tokens, m->embed_scale, T, W, m->V, dt, st));
+  bool h_ready = false;
   for (int l = 0; l < m->L; ++l) {
     const UmbSeqLayer& ly = m->layers[l];
+    const UmbSeqLayer* nl = l + 1 < m->L ? &m->layers[l + 1] : nullptr;
     const int ld = ly.proj.N;
-    SEQ_TRY(sublayer_input(m, ws, s, ly.norm1, ly.canon1, ly.canon_state1, st));
+    SEQ_TRY(sublayer_input(m, ws, s, ly.norm1, ly.canon1, ly.canon_state1, h_ready, st));
     SEQ_TRY(lin(ly.proj, ws->proj, ws->h, T, 0, dt, st));
     if (ly.kind == UMB_MIX_POOLED_WINDOW) {
       const int H = ly.heads, G = ly.kv_heads, D = ly.dim;
@@ -127,11 +147,13 @@ extern "C" int umb_seq_forward(const UmbSeqModel* m, const UmbSeqWork* ws, const
     }
     SEQ_TRY(lin(ly.out, ws->y, ws->mix, T, 0, dt, st));
     const void* next = ly.has_mlp ? ly.norm2 : first_norm_of(m, l + 1);
-    SEQ_TRY(umb_seq_resid_norm(ws->x, ws->h, ws->y, ly.norm1b, next, T, W, groups, eps, dt, st));
+    SEQ_TRY(seam(m, ws, s, ly.norm1b, next, ly.has_mlp ? ly.canon2 : (nl ? nl->canon1 : nullptr),
+                 ly.has_mlp ? ly.canon_state2 : (nl ? nl->canon_state1 : nullptr), &h_ready, st));
     if (ly.has_mlp) {
-      SEQ_TRY(sublayer_input(m, ws, s, ly.norm2, ly.canon2, ly.canon_state2, st));
+      SEQ_TRY(sublayer_input(m, ws, s, ly.norm2, ly.canon2, ly.canon_state2, h_ready, st));
       SEQ_TRY(feed_forward(m, ly, ws, s, st));
-      SEQ_TRY(umb_seq_resid_norm(ws->x, ws->h, ws->y, ly.norm2b, first_norm_of(m, l + 1), T, W, groups, eps, dt, st));
+      SEQ_TRY(seam(m, ws, s, ly.norm2b, first_norm_of(m, l + 1), nl ? nl->canon1 : nullptr, nl ? nl->canon_state1 : nullptr,
+                   &h_ready, st));
     }
     if (s->trace) {
       if (hipMemcpyAsync(s->trace + (long)l * T * W, ws->x, (size_t)T * W * sizeof(float), hipMemcpyDeviceToDevice, st) != hipSuccess)
