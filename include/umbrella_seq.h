@@ -83,7 +83,9 @@ int umb_canon_step(void* h, const float* x, const void* w, float* state, const i
                    int taps, int dtype, umb_stream_t stream);
 
 /* The seam x <- x + group_norm(y) * w_post followed by that convolution, for steps of one token per sequence, in one
- * launch: h = canon(x), the state row of the token's position is overwritten with the new x.  W / groups <= 8192. */
+ * launch: h = canon(x), the state row of the token's position is overwritten with the new x.  Covers groups == 1 and
+ * groups whose length is a multiple of 256 (umb_seq_resid_canon_step_ok: 1 / 0, no stream). */
+int umb_seq_resid_canon_step_ok(int W, int groups);
 int umb_seq_resid_canon_step(float* x, void* h, const float* y, const void* w_post, const void* canon, float* state,
                              const int* pos, const int* slot, int T, int W, int groups, int taps, float eps, int dtype,
                              umb_stream_t stream);

@@ -98,6 +98,13 @@ def test_grouped_linear_walks_a_tile_list(lib, dtype):
     act = torch.zeros(150, N, dtype=dtype, device="cuda:0")
     _lib.seq_call("umb_seq_linear_grouped", act, dev(x), dev(w), i32(tiles), len(tiles), 64, 2 * N * K, 2 * N, K, 2, code)
     assert close(act, torch.nn.functional.silu(want[:, :N]) * want[:, N:], tol)
+    small = [(3, 10, 16), (0, 26, 1), (1, 27, 5), (2, 0, 0)]          # tiles of up to 16 rows: one output tile per workgroup
+    out.zero_()
+    _lib.seq_call("umb_seq_linear_grouped", out, dev(x), dev(w), i32(small), len(small), 16, 2 * N * K, 2 * N, K, 0, code)
+    g16 = torch.zeros(150, dtype=torch.long)
+    g16[10:26], g16[26], g16[27:32] = 3, 0, 1
+    w16 = torch.einsum("tk,tnk->tn", x.double(), w.double()[g16])
+    assert close(out[10:32], w16[10:32], tol) and float(out[:10].abs().max()) == 0.0 and float(out[32:].abs().max()) == 0.0
     if dtype != torch.float32:               # tiles of up to 128 rows on the LDS-staged kernel
         big = [(1, 0, 128), (3, 128, 22), (0, 0, 0)]
         grp[:128], grp[128:150] = 1, 3
@@ -164,6 +171,26 @@ def test_input_convolution_batch_of_unequal_sequences(lib):
         got["a"].append(h[:na].clone()), got["b"].append(h[na:].clone())
     assert close(torch.cat(got["a"]), O.conv_input(xa.double(), w.double()), 1e-6)
     assert close(torch.cat(got["b"]), O.conv_input(xb.double(), w.double()), 1e-6)
+
+
+@pytest.mark.parametrize("taps,W,groups", [(1, 40, 1), (2, 300, 1), (4, 2048, 1), (3, 1024, 2), (7, 520, 1)])
+def test_seam_with_convolution_in_one_launch(lib, taps, W, groups):
+    """single-token steps: x += norm(y) * w, h = conv(x), state update -- against the oracle over a whole sequence"""
+    from oracle import seqmix as O
+    from umbrella_amd import _lib
+    assert lib.umb_seq_resid_canon_step_ok(W, groups) == 1 and lib.umb_seq_resid_canon_step_ok(300, 3) == 0
+    g = torch.Generator().manual_seed(W)
+    n, eps = 9, 1e-5
+    x0, y = torch.randn(n, W, generator=g), torch.randn(n, W, generator=g)
+    w_post, w = 1 + 0.1 * torch.randn(W, generator=g), torch.randn(W, taps, generator=g)
+    x_want = x0.double() + O.group_rms_norm(y.double(), w_post.double(), groups, eps)
+    h_want = O.conv_input(x_want, w.double())
+    state = torch.full((2, max(taps - 1, 1), W), 1e6, dtype=torch.float32, device="cuda:0")
+    wd, wp = dev(w), dev(w_post)
+    for t in range(n):
+        x, h = dev(x0[t:t + 1]), torch.zeros(1, W, dtype=torch.float32, device="cuda:0")
+        _lib.seq_call("umb_seq_resid_canon_step", x, h, dev(y[t:t + 1]), wp, wd, state, i32([t]), i32([1]), 1, W, groups, taps, eps, 2)
+        assert close(x, x_want[t:t + 1], 1e-6) and close(h, h_want[t:t + 1], 1e-5), t
 
 
 # ------------------------------------------------------------------ feed-forward pieces

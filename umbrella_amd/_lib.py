@@ -259,6 +259,7 @@ SEQ_SIGNATURES = {
     "umb_canon_update": [_P, _P, _P, _P, _P, _P, _I, _I, _I],
     "umb_canon_step": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I],
     "umb_seq_resid_canon_step": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I],
+    "umb_seq_resid_canon_step_ok": [_I, _I],
     "umb_polynorm": [_P, _P, _P, _I, _I, _F, _I],
     "umb_moe_route": [_P, _P, _P, _I, _I, _I],
     "umb_moe_plan": [_P, _P, _P, _I, _I, _I, _I, _I],
@@ -284,7 +285,7 @@ SEQ_SIGNATURES = {
     "umb_sample_rows": [_P, _P, _I, _I, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P],
     "umb_seq_version": [],
 }
-_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok"}          # predicates: no stream argument, the value is the answer
+_SEQ_NO_STREAM = {"umb_lat_attend_tiled_ok", "umb_seq_resid_canon_step_ok"}          # predicates: no stream argument, the value is the answer
 _seq_lib = None
 
 

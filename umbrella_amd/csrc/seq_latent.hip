@@ -17,8 +17,8 @@
 
 static inline bool lat_kv_ok(const UmbPagedKV* kv) { return kv && kv->k && kv->pages && kv->page >= 1 && kv->max_pages >= 1; }
 
-// ---- norms of the two latents, rotation of the shared key part, cache append.  One wave per (token, part): part 0 = the
-// query latent, part 1 = the key/value latent + rotated key.
+// ---- norms of the two latents, rotation of the shared key part, cache append.  One workgroup per (token, part): part 0 =
+// the query latent, part 1 = the key/value latent + rotated key.
 template <typename P>
 __global__ __launch_bounds__(256) void lat_prep_kernel(typename El<P>::type* __restrict__ cq, UmbPagedKV kv,
                                                        const float* __restrict__ proj, int ld,
@@ -27,26 +27,26 @@ __global__ __launch_bounds__(256) void lat_prep_kernel(typename El<P>::type* __r
                                                        const int* __restrict__ slot, const float* __restrict__ freq, int T,
                                                        int q_rank, int kv_rank, int rot_dim, int rot_dims, float eps) {
   typedef typename El<P>::type E;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const long id = (long)blockIdx.x * 4 + wave;
-  if (id >= 2L * T) return;
-  const int t = (int)(id >> 1), part = (int)(id & 1);
+  __shared__ float red[8];
+  const int lane = threadIdx.x;
+  const int t = blockIdx.x >> 1, part = blockIdx.x & 1;
   const float* src = proj + (long)t * ld + (part ? q_rank : 0);
   const int n = part ? kv_rank : q_rank;
   float ss = 0.f;
-  for (int i = lane; i < n; i += 64) { const float v = src[i]; ss += v * v; }
-  ss = wave_sum(ss);
+#pragma unroll 4
+  for (int i = lane; i < n; i += 256) { const float v = src[i]; ss += v * v; }
+  ss = block_sum<256>(ss, red);
   const float f = 1.f / sqrtf(ss / (float)n + eps);
   if (!part) {
-    for (int i = lane; i < n; i += 64) stf<P>(cq + (long)t * q_rank + i, src[i] * f * ldf<P>(w_q + i));
+    for (int i = lane; i < n; i += 256) stf<P>(cq + (long)t * q_rank + i, src[i] * f * ldf<P>(w_q + i));
     return;
   }
   const int p = pos[t];
   E* row = reinterpret_cast<E*>(kv.k) + pkv_tok(kv, slot[t], p, 0, 1, kv_rank + rot_dim);
-  for (int i = lane; i < n; i += 64) stf<P>(row + i, src[i] * f * ldf<P>(w_kv + i));
+  for (int i = lane; i < n; i += 256) stf<P>(row + i, src[i] * f * ldf<P>(w_kv + i));
   const float* kr = src + kv_rank;
   const float pf = (float)p;
-  for (int m = lane; m < (rot_dim + 1) / 2; m += 64) {
+  for (int m = lane; m < (rot_dim + 1) / 2; m += 256) {
     const int d0 = 2 * m, d1 = 2 * m + 1;
     float u = kr[d0], v = d1 < rot_dim ? kr[d1] : 0.f;
     if (d1 < rot_dims) {
@@ -245,7 +245,7 @@ extern "C" int umb_lat_prep(void* cq, const UmbPagedKV* kv, const float* proj, i
     return UMB_EINVAL;
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
-    hipLaunchKernelGGL(lat_prep_kernel<P>, dim3((unsigned)((2L * T + 3) / 4)), dim3(256), 0, st, (E*)cq, *kv, proj, ld,
+    hipLaunchKernelGGL(lat_prep_kernel<P>, dim3((unsigned)(2L * T)), dim3(256), 0, st, (E*)cq, *kv, proj, ld,
                        (const E*)w_q, (const E*)w_kv, pos, slot, freq, T, q_rank, kv_rank, rot_dim, rot_dims, eps);
   })
   UMB_LAUNCH_CHECK();

@@ -391,7 +391,7 @@ extern "C" int umb_seq_linear_batched(void* out, const void* x, const void* w, i
 extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, const int* tiles, int max_tiles, int tile_rows,
                                       long gs, int N, int K, int epi, int dtype, hipStream_t st) {
   if (max_tiles < 1 || max_tiles > 65535 || N < 1 || K < 1 || epi < 0 || epi > 2 || !out || !x || !w || !tiles ||
-      (tile_rows != 64 && tile_rows != 128))
+      (tile_rows != 16 && tile_rows != 64 && tile_rows != 128))
     return UMB_EINVAL;
   if (epi == EPI_SILU_MUL) {
     if (N & 1) return UMB_EINVAL;
@@ -402,6 +402,12 @@ extern "C" int umb_seq_linear_grouped(void* out, const void* x, const void* w, c
     if (dtype == UMB_SEQ_F32 || K % 8 || gs % 8) return UMB_EINVAL;
     if (dtype == UMB_SEQ_BF16) return launch_wide<BF16>(out, x, w, nullptr, 128, N, K, epi, st, ext, max_tiles);
     return launch_wide<F16>(out, x, w, nullptr, 128, N, K, epi, st, ext, max_tiles);
+  }
+  if (tile_rows == 16) {                   // a few rows in all (decoding): one 16-row output tile per workgroup, many workgroups
+    DISPATCH_SEQ_DTYPE(dtype, {
+      if (K % 8 == 0 && gs % 8 == 0) return launch_tt<P, 1, 1, true>(out, x, w, nullptr, 16, N, K, epi, st, ext, max_tiles);
+      return launch_tt<P, 1, 1, false>(out, x, w, nullptr, 16, N, K, epi, st, ext, max_tiles);
+    })
   }
   DISPATCH_SEQ_DTYPE(dtype, {
     if (K % 8 == 0 && gs % 8 == 0) {

@@ -41,7 +41,7 @@ static int seam(const UmbSeqModel* m, const UmbSeqWork* ws, const UmbSeqStep* s,
                 const void* next_canon, float* next_state, bool* h_ready, hipStream_t st) {
   const int T = s->T, W = m->W;
   *h_ready = false;
-  if (!w_next && next_canon && s->max_len == 1 && W / m->groups <= 8192) {
+  if (!w_next && next_canon && s->max_len == 1 && umb_seq_resid_canon_step_ok(W, m->groups)) {
     *h_ready = true;
     return umb_seq_resid_canon_step(ws->x, ws->h, ws->y, w_post, next_canon, next_state, s->pos, s->slot, T, W, m->groups,
                                     m->canon_taps, m->eps, m->dtype, st);
@@ -69,7 +69,8 @@ static int feed_forward(const UmbSeqModel* m, const UmbSeqLayer& ly, const UmbSe
       return UMB_EINVAL;
     const long pairs = (long)T * top;
     // many rows per expert (prompts): tiles of 128 rows on the LDS-staged kernel; few (decoding): tiles of 64, weights streamed
-    const int tr = (dt != UMB_SEQ_F32 && pairs >= 64L * E && W % 8 == 0 && F % 8 == 0) ? 128 : 64;
+    // a handful of rows in all: tiles of 16, one output tile per workgroup
+    const int tr = (dt != UMB_SEQ_F32 && pairs >= 64L * E && W % 8 == 0 && F % 8 == 0) ? 128 : (pairs <= 64 ? 16 : 64);
     const int max_tiles = (int)((pairs + tr - 1) / tr) + E;
     if (max_tiles > ws->moe_max_tiles) return UMB_EINVAL;
     if (ly.s_gu.w) {                                                           // the shared expert sees every token

@@ -114,17 +114,12 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(float* __restrict__ x, 
 // ---- long groups (more than 16 elements per lane of one wave): a whole workgroup owns one (row, group), its 256 threads hold
 // EPT elements each in registers, the two sums of squares go through LDS.  A decode step has few rows: one wave per row would
 // leave a 4096-wide row to 64 lanes and three dependent passes over memory.
-// CANON: the seam is followed by the causal convolution in front of the next sublayer, for a step of ONE token per sequence:
-// h = x' + sum_j w[c][j] x'(p - taps + 1 + j), earlier positions read from the sequence's state rows ((p - k) % (taps - 1)),
-// and the state row of p is overwritten with x' by the thread that read it -- seam, convolution and state update in one launch.
-template <typename P, int EPT, bool CANON>
+template <typename P, int EPT>
 __global__ __launch_bounds__(256) void resid_norm_block_kernel(float* __restrict__ x, typename El<P>::type* __restrict__ h,
                                                                const float* __restrict__ y,
                                                                const typename El<P>::type* __restrict__ w_post,
                                                                const typename El<P>::type* __restrict__ w_next, int W, int groups,
-                                                               float eps, const typename El<P>::type* __restrict__ canon,
-                                                               float* __restrict__ state, const int* __restrict__ pos,
-                                                               const int* __restrict__ slot, int taps) {
+                                                               float eps) {
   __shared__ float red[8];
   const int t = blockIdx.x, grp = blockIdx.y, gs = W / groups;
   const long o = (long)t * W + (long)grp * gs;
@@ -148,24 +143,7 @@ __global__ __launch_bounds__(256) void resid_norm_block_kernel(float* __restrict
     xv[e] = xv[e] + yv[e] * f * wp[e];
     if (i < gs) { x[o + i] = xv[e]; s2 += xv[e] * xv[e]; }
   }
-  if constexpr (CANON) {
-    const int p = pos[t], S = taps - 1;
-    float* st = state + (long)slot[t] * S * W + (long)grp * gs;
-#pragma unroll
-    for (int e = 0; e < EPT; ++e) {
-      const int i = threadIdx.x + 256 * e;
-      if (i >= gs) continue;
-      const typename El<P>::type* wc = canon + ((long)grp * gs + i) * taps;
-      float a = xv[e] * (1.f + ldf<P>(wc + S));
-      for (int k = 1; k <= S; ++k) {
-        const bool in = p - k >= 0;
-        const float v = st[(long)((in ? p - k : 0) % S) * W + i];
-        a += in ? ldf<P>(wc + S - k) * v : 0.f;
-      }
-      stf<P>(h + o + i, a);
-      if (S > 0) st[(long)(p % S) * W + i] = xv[e];
-    }
-  } else {
+  {
     if (!w_next) return;
     s2 = block_sum<256>(s2, red);
     const float f2 = 1.f / sqrtf(s2 / (float)gs + eps);
@@ -203,6 +181,56 @@ __global__ __launch_bounds__(256) void group_norm_block_kernel(float* __restrict
     if (out_f32) out_f32[o + i] = v;
     if (out_dt) stf<P>(out_dt + o + i, v);
   }
+}
+
+// The seam of a step of ONE token per sequence, followed by the next sublayer's causal convolution and its state update.
+// Workgroup = (token, 256 channels); every workgroup of a token first sums the squares of the token's whole group of y by
+// itself (a row is a few KiB: cheaper than a second launch), then each thread finishes one channel: x' = x + y f w_post,
+// h = x' + sum_j w[c][j] x'(p - taps + 1 + j) with the earlier positions read from the sequence's state rows
+// ((p - k) % (taps - 1)), and the state row of p overwritten with x' by the thread that read it.  The loads of the taps do not
+// depend on one another (TAPS > 0: unrolled).
+template <typename P, int TAPS>
+__global__ __launch_bounds__(256) void seam_canon_step_kernel(float* __restrict__ x, typename El<P>::type* __restrict__ h,
+                                                              const float* __restrict__ y,
+                                                              const typename El<P>::type* __restrict__ w_post,
+                                                              const typename El<P>::type* __restrict__ canon,
+                                                              float* __restrict__ state, const int* __restrict__ pos,
+                                                              const int* __restrict__ slot, int W, int groups, float eps,
+                                                              int taps_rt) {
+  __shared__ float red[8];
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x, gs = W / groups;
+  const int grp = (blockIdx.y * 256) / gs;                    // the workgroup's channels lie in one group
+  const float* yr = y + (long)t * W + (long)grp * gs;
+  float ss = 0.f;
+#pragma unroll 8
+  for (int i = threadIdx.x; i < gs; i += 256) { const float v = yr[i]; ss += v * v; }
+  ss = block_sum<256>(ss, red);
+  if (c >= W) return;
+  const float f = 1.f / sqrtf(ss / (float)gs + eps);
+  const int taps = TAPS > 0 ? TAPS : taps_rt, S = taps - 1;
+  const int p = pos[t];
+  float* st = state + (long)slot[t] * S * W + c;
+  const typename El<P>::type* wc = canon + (long)c * taps;
+  const float xn = x[(long)t * W + c] + y[(long)t * W + c] * f * ldf<P>(w_post + c);
+  x[(long)t * W + c] = xn;
+  float a = xn * (1.f + ldf<P>(wc + S));
+  if constexpr (TAPS > 0) {
+    float v[TAPS], wk[TAPS];
+#pragma unroll
+    for (int k = 1; k < TAPS; ++k) {
+      v[k] = st[(long)((p - k >= 0 ? p - k : 0) % (TAPS - 1)) * W];
+      wk[k] = ldf<P>(wc + (TAPS - 1) - k);
+    }
+#pragma unroll
+    for (int k = 1; k < TAPS; ++k) a += p - k >= 0 ? wk[k] * v[k] : 0.f;
+  } else {
+    for (int k = 1; k <= S; ++k) {
+      const float v = st[(long)((p - k >= 0 ? p - k : 0) % S) * W];
+      a += p - k >= 0 ? ldf<P>(wc + S - k) * v : 0.f;
+    }
+  }
+  stf<P>(h + (long)t * W + c, a);
+  if (S > 0) st[(long)(p % S) * W] = xn;
 }
 
 static inline bool norm_args_ok(int T, int W, int groups) { return T >= 1 && W >= 1 && groups >= 1 && W % groups == 0; }
@@ -248,13 +276,11 @@ extern "C" int umb_seq_resid_norm(float* x, void* h, const float* y, const void*
     const dim3 grid(T, (groups + 3) / 4);
     const int gs = W / groups;
     if (per_lane > 16 && gs <= 2048)
-      hipLaunchKernelGGL((resid_norm_block_kernel<P, 8, false>), dim3(T, groups), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
-                         (const E*)w_next, W, groups, eps, (const E*)nullptr, (float*)nullptr, (const int*)nullptr,
-                         (const int*)nullptr, 0);
+      hipLaunchKernelGGL((resid_norm_block_kernel<P, 8>), dim3(T, groups), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
+                         (const E*)w_next, W, groups, eps);
     else if (per_lane > 16 && gs <= 8192)
-      hipLaunchKernelGGL((resid_norm_block_kernel<P, 32, false>), dim3(T, groups), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
-                         (const E*)w_next, W, groups, eps, (const E*)nullptr, (float*)nullptr, (const int*)nullptr,
-                         (const int*)nullptr, 0);
+      hipLaunchKernelGGL((resid_norm_block_kernel<P, 32>), dim3(T, groups), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
+                         (const E*)w_next, W, groups, eps);
     else if (per_lane <= 4)
       hipLaunchKernelGGL((resid_norm_kernel<P, 4>), grid, dim3(256), 0, st, x, (E*)h, y, (const E*)w_post, (const E*)w_next, W,
                          groups, eps);
@@ -269,25 +295,31 @@ extern "C" int umb_seq_resid_norm(float* x, void* h, const float* y, const void*
   return UMB_OK;
 }
 
+extern "C" int umb_seq_resid_canon_step_ok(int W, int groups) {
+  return W >= 1 && groups >= 1 && W % groups == 0 && (groups == 1 || (W / groups) % 256 == 0);
+}
+
 extern "C" int umb_seq_resid_canon_step(float* x, void* h, const float* y, const void* w_post, const void* canon, float* state,
                                         const int* pos, const int* slot, int T, int W, int groups, int taps, float eps, int dtype,
                                         hipStream_t st) {
   if (!norm_args_ok(T, W, groups) || !x || !h || !y || !w_post || !canon || !pos || !slot || taps < 1 || (taps > 1 && !state) ||
-      W / groups > 8192)
+      !umb_seq_resid_canon_step_ok(W, groups))
     return UMB_EINVAL;
-  const int gs = W / groups;
+  const dim3 grid(T, (W + 255) / 256);
+#define SEAM_LAUNCH(TAPS)                                                                                                  \
+  hipLaunchKernelGGL((seam_canon_step_kernel<P, TAPS>), grid, dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,             \
+                     (const E*)canon, state, pos, slot, W, groups, eps, taps)
   DISPATCH_SEQ_DTYPE(dtype, {
     typedef typename El<P>::type E;
-    if (gs <= 1024)
-      hipLaunchKernelGGL((resid_norm_block_kernel<P, 4, true>), dim3(T, groups), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
-                         (const E*)nullptr, W, groups, eps, (const E*)canon, state, pos, slot, taps);
-    else if (gs <= 2048)
-      hipLaunchKernelGGL((resid_norm_block_kernel<P, 8, true>), dim3(T, groups), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
-                         (const E*)nullptr, W, groups, eps, (const E*)canon, state, pos, slot, taps);
-    else
-      hipLaunchKernelGGL((resid_norm_block_kernel<P, 32, true>), dim3(T, groups), dim3(256), 0, st, x, (E*)h, y, (const E*)w_post,
-                         (const E*)nullptr, W, groups, eps, (const E*)canon, state, pos, slot, taps);
+    switch (taps) {
+      case 2: SEAM_LAUNCH(2); break;
+      case 3: SEAM_LAUNCH(3); break;
+      case 4: SEAM_LAUNCH(4); break;
+      case 5: SEAM_LAUNCH(5); break;
+      default: SEAM_LAUNCH(0); break;
+    }
   })
+#undef SEAM_LAUNCH
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }

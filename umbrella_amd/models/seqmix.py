@@ -219,7 +219,7 @@ class SeqMixLM(LLMBase):
             setattr(ws, k, b[k].data_ptr())
         if top:
             pairs = T * top
-            tiles = (pairs + 63) // 64 + max(ly.experts for ly in c.layers)
+            tiles = (pairs + 15) // 16 + max(ly.experts for ly in c.layers)          # the smallest tile size the forward picks
             b.update(moe_sel=torch.zeros(pairs, dtype=i32, device=dev), moe_wt=torch.zeros(pairs, dtype=f32, device=dev),
                      moe_pos=torch.zeros(pairs, dtype=i32, device=dev), moe_tiles=torch.zeros(tiles, 3, dtype=i32, device=dev),
                      moe_xs=torch.zeros(pairs, c.width, dtype=dt, device=dev), moe_act=torch.zeros(pairs, eff, dtype=dt, device=dev),
