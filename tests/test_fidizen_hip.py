@@ -367,12 +367,15 @@ MFMA_CASES = [  # H, D, R, E, q_rank, kv_rank, window, rot_dims, page: key rows 
     (16, 8, 8, 8, 16, 64, 33, 8, 5), (3, 8, 24, 12, 16, 80, 1, 4, 3), (8, 16, 0, 16, 8, 16, 20, 0, 7)]
 
 
+@pytest.mark.parametrize("single", ["vector", "matrix"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("H,D,R,E,q_rank,kv_rank,window,rot_dims,page", MFMA_CASES)
-def test_latent_attention_on_the_matrix_pipe(lib, dtype, H, D, R, E, q_rank, kv_rank, window, rot_dims, page):
+def test_latent_attention_on_the_matrix_pipe(lib, monkeypatch, single, dtype, H, D, R, E, q_rank, kv_rank, window, rot_dims, page):
     """16-bit storage: prompt portions of 16 tokens and more take the matrix-pipe kernel (tiles that start inside a window,
-    end before a full tile, span pages), shorter ones the scalar kernel; both against the oracle and against each other"""
+    end before a full tile, span pages); shorter ones the vector-pipe kernel or, from a few dozen tokens a step (here: forced),
+    the matrix-pipe kernel whose query tile is sixteen heads of one token; all against the oracle and against each other"""
     from umbrella_amd import _lib
+    monkeypatch.setenv("UMB_LAT_DEC_MIN", "0" if single == "matrix" else "1000000")
     assert lib.umb_lat_attend_tiled_ok(H, kv_rank, R, _lib.seq_dtype_code(dtype)) == 1
     width, n = 40, 100
     w = _lat_weights(width, H, D, R, E, q_rank, kv_rank, seed=H + kv_rank)
@@ -397,15 +400,17 @@ def _loud(n, width, rows, seed):
     return X
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_latent_window_edges_and_far_keys_with_loud_rows(lib, dtype):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_latent_window_edges_and_far_keys_with_loud_rows(lib, monkeypatch, dtype):
     """loud keys just inside and just outside the window of the last positions, at a page border and far back, in a prompt
     and in token-by-token decoding; the softmax spans hundreds of keys"""
+    if dtype == torch.float16:                       # this run decodes single tokens on the matrix pipe
+        monkeypatch.setenv("UMB_LAT_DEC_MIN", "0")
     H, D, R, E, q_rank, kv_rank, window, page = 4, 16, 8, 16, 24, 48, 150, 32
     width, n = 48, 260
     w = _lat_weights(width, H, D, R, E, q_rank, kv_rank, seed=5)
     kw = dict(H=H, D=D, R=R, E=E, kv_rank=kv_rank, window=window, rot_dims=8, base=1000.0, scale=0.2, eps=1e-5)
-    tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+    tol = F32_TOL if dtype == torch.float32 else (BF16_TOL if dtype == torch.bfloat16 else 1e-2)
     for rows in ([n - window], [n - window - 1], [n - 1 - window, 3], [0, 31, 32, n - window + 1], [n - 20 - window, n - 21 - window]):
         X = _loud(n, width, rows, seed=len(rows))
         want = _lat_oracle(X, w, dtype, **kw)
@@ -553,6 +558,34 @@ def test_model_unequal_batch_equals_each_alone(lib, dtype):
     alone["z"] = m.forward_batch([("z0", late)], want=[list(range(len(late)))]).clone()
     for k in seqs:
         assert rel_err(torch.cat(got[k]), alone[k]) < tol, k
+
+
+def test_model_sixty_sequences_decoded_together(lib):
+    """bf16: sixty requests of different lengths, prefilled in one ragged step and decoded together for a few steps (steps of
+    sixty single tokens take the matrix-pipe kernel for single tokens), against each request alone"""
+    from fidizen_helpers import CONFIGS, build
+    cfgd = _few_experts(CONFIGS["wide"])
+    m, _ = build(cfgd, torch.bfloat16, seed=5, page=8, batch=61, max_tokens=4000)
+    V = cfgd["vocab"]
+    seqs = {k: tokens(4 + (7 * k) % 40, V, 100 + k) for k in range(60)}
+    for k in seqs:
+        m.open(k)
+    got = {k: [] for k in seqs}
+    out = m.forward_batch([(k, t[:-3]) for k, t in seqs.items()]).clone()          # the last row of each
+    for i, k in enumerate(seqs):
+        got[k].append(out[i:i + 1])
+    for step in range(3):
+        out = m.forward_batch([(k, [t[len(t) - 3 + step]]) for k, t in seqs.items()]).clone()
+        for i, k in enumerate(seqs):
+            got[k].append(out[i:i + 1])
+    worst = 0.0
+    for k, t in list(seqs.items())[::7]:
+        m.open("solo")
+        n = len(t)
+        alone = m.forward_batch([("solo", t)], want=[[n - 4, n - 3, n - 2, n - 1]]).clone()
+        m.close("solo")
+        worst = max(worst, rel_err(torch.cat(got[k]), alone))
+    assert worst < 3e-2, worst
 
 
 def test_model_long_decoding_past_the_window_and_first_tokens(lib):

@@ -14,6 +14,7 @@
 // pos * freq[i] in fp32 through the full-range sincosf; pairs (2i, 2i+1) of the first rot_dims features of the rotated part
 // turn, the rest pass.
 #include "seq_common.h"
+#include <cstdlib>
 
 static inline bool lat_kv_ok(const UmbPagedKV* kv) { return kv && kv->k && kv->pages && kv->page >= 1 && kv->max_pages >= 1; }
 
@@ -237,74 +238,6 @@ __global__ __launch_bounds__(NW * 64) void lat_attend_kernel(typename El<P>::typ
   }
 }
 
-extern "C" int umb_lat_prep(void* cq, const UmbPagedKV* kv, const float* proj, int ld, const void* w_q, const void* w_kv,
-                            const int* pos, const int* slot, const float* freq, int T, int q_rank, int kv_rank, int rot_dim,
-                            int rot_dims, float eps, int dtype, hipStream_t st) {
-  if (T < 1 || q_rank < 1 || kv_rank < 1 || rot_dim < 0 || rot_dims < 0 || rot_dims > rot_dim || (rot_dims & 1) || !cq ||
-      !lat_kv_ok(kv) || !proj || !w_q || !w_kv || !pos || !slot || (rot_dims && !freq) || ld < q_rank + kv_rank + rot_dim)
-    return UMB_EINVAL;
-  DISPATCH_SEQ_DTYPE(dtype, {
-    typedef typename El<P>::type E;
-    hipLaunchKernelGGL(lat_prep_kernel<P>, dim3((unsigned)(2L * T)), dim3(256), 0, st, (E*)cq, *kv, proj, ld,
-                       (const E*)w_q, (const E*)w_kv, pos, slot, freq, T, q_rank, kv_rank, rot_dim, rot_dims, eps);
-  })
-  UMB_LAUNCH_CHECK();
-  return UMB_OK;
-}
-
-extern "C" int umb_lat_qsplit(void* qn, float* qa, const float* q, const int* pos, const float* freq, int T, int H, int D, int R,
-                              int kv_rank, int rot_dims, int dtype, hipStream_t st) {
-  if (T < 1 || H < 1 || D < 1 || R < 0 || kv_rank < 1 || rot_dims < 0 || rot_dims > R || (rot_dims & 1) || !qn || !qa || !q ||
-      !pos || (rot_dims && !freq))
-    return UMB_EINVAL;
-  const long n = (long)T * H * (D + (R + 1) / 2);
-  DISPATCH_SEQ_DTYPE(dtype, {
-    typedef typename El<P>::type E;
-    hipLaunchKernelGGL(lat_qsplit_kernel<P>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (E*)qn, qa, q, pos, freq, T, H,
-                       D, R, kv_rank, rot_dims);
-  })
-  UMB_LAUNCH_CHECK();
-  return UMB_OK;
-}
-
-extern "C" int umb_lat_attend(void* out, const float* qa, const UmbPagedKV* kv, const void* sink, const int* pos, const int* slot,
-                              int T, int H, int kv_rank, int rot_dim, int window, float scale, int dtype, hipStream_t st) {
-  if (T < 1 || H < 1 || kv_rank < 1 || kv_rank > 64 * LAT_MAXC || rot_dim < 0 || window < 1 || !out || !qa || !lat_kv_ok(kv) ||
-      !pos || !slot)
-    return UMB_EINVAL;
-  const int Dk = kv_rank + rot_dim, Dp = (Dk + 3) & ~3;
-  // heads of one workgroup: all of them share the keys, so as many as the register budget of the partial sums allows
-  const int nc = (kv_rank + 63) / 64;
-  int rh = nc <= 2 ? 8 : (nc <= 4 ? 4 : 2);
-  while (rh > 1 && rh / 2 >= H) rh >>= 1;
-  const int hb = (H + rh - 1) / rh;
-  const dim3 grid(T, hb);
-  int nw = (long)T * hb < 1024 ? 16 : 4;
-  auto lds_of = [&](int w) { return ((size_t)w * rh * Dp + (size_t)w * 2 * rh + (size_t)w * (rh * 64 + 128)) * sizeof(float); };
-  if (nw == 16 && lds_of(16) > 128 * 1024) nw = 4;
-  if (lds_of(nw) > 160 * 1024) return UMB_EINVAL;
-  const size_t lds = lds_of(nw);
-#define LAT_LAUNCH(RH, NC, NW)                                                                                            \
-  do {                                                                                                                    \
-    if (ensure_dynamic_lds<lat_attend_kernel<P, RH, NC, NW>>(lds) != UMB_OK) return UMB_EHIP;                             \
-    hipLaunchKernelGGL((lat_attend_kernel<P, RH, NC, NW>), grid, dim3(NW * 64), lds, st, (E*)out, qa, *kv, (const E*)sink, \
-                       pos, slot, T, H, kv_rank, rot_dim, window, scale);                                                 \
-  } while (0)
-#define LAT_NW(RH, NC)                                                                                                    \
-  if (nw == 16) LAT_LAUNCH(RH, NC, 16); else LAT_LAUNCH(RH, NC, 4)
-  DISPATCH_SEQ_DTYPE(dtype, {
-    typedef typename El<P>::type E;
-    if (nc <= 1) { if (rh == 8) { LAT_NW(8, 1); } else if (rh == 4) { LAT_NW(4, 1); } else if (rh == 2) { LAT_NW(2, 1); } else { LAT_NW(1, 1); } }
-    else if (nc <= 2) { if (rh == 8) { LAT_NW(8, 2); } else if (rh == 4) { LAT_NW(4, 2); } else if (rh == 2) { LAT_NW(2, 2); } else { LAT_NW(1, 2); } }
-    else if (nc <= 4) { if (rh == 4) { LAT_NW(4, 4); } else if (rh == 2) { LAT_NW(2, 4); } else { LAT_NW(1, 4); } }
-    else { if (rh == 2) { LAT_NW(2, 8); } else { LAT_NW(1, 8); } }
-  })
-#undef LAT_NW
-#undef LAT_LAUNCH
-  UMB_LAUNCH_CHECK();
-  return UMB_OK;
-}
-
 // ---- prompt attention on the matrix pipe (16-bit storage; Dk a multiple of 8, kv_rank a multiple of 16).
 // Workgroup = (16 consecutive positions of one sequence, a block of 4 HPW heads); wave w owns HPW heads and walks the tile's
 // keys -- from the first position's window start to the last position -- in steps of 32, alone (no workgroup barrier).
@@ -366,7 +299,7 @@ __global__ __launch_bounds__(256) void lat_attend_mfma_kernel(u16* __restrict__ 
     m_run[hh] = -INFINITY;
     l_run[hh] = 0.f;
   }
-  const int pieces = 32 * (Dc >> 3);                 // 16-byte pieces of the step's value tile
+  const int nch = Dc >> 3;                            // 16-byte chunks of a value row
   for (int base = 0; base < total; base += 32) {
     if (lane < 32) {
       const int kx = base + lane;
@@ -374,11 +307,23 @@ __global__ __launch_bounds__(256) void lat_attend_mfma_kernel(u16* __restrict__ 
     }
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    for (int p = lane; p < pieces; p += 64) {
-      const int m = p / (Dc >> 3), dp = (p % (Dc >> 3)) * 8;
-      const long off = offs[m];
-      const u32x4 v = off >= 0 ? *reinterpret_cast<const u32x4*>(kbase + off + dp) : u32x4{0u, 0u, 0u, 0u};
-      *reinterpret_cast<u32x4*>(v_s + m * LD + dp) = v;
+    {
+      // lane = (key row m, parity of the 16-byte chunk); eight chunks of the row in flight before any is written
+      const int m = lane & 31, c0 = lane >> 5;
+      const long offm = offs[m];
+      for (int cb = 0; cb < nch; cb += 16) {
+        u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int ch = cb + c0 + 2 * u;
+          v[u] = (ch < nch && offm >= 0) ? *reinterpret_cast<const u32x4*>(kbase + offm + 8 * ch) : u32x4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int ch = cb + c0 + 2 * u;
+          if (ch < nch) *reinterpret_cast<u32x4*>(v_s + m * LD + 8 * ch) = v[u];
+        }
+      }
     }
     f32x4 sc[HPW][2];
 #pragma unroll
@@ -473,6 +418,168 @@ __global__ __launch_bounds__(256) void lat_attend_mfma_kernel(u16* __restrict__ 
   }
 }
 
+// ---- single tokens on the matrix pipe (16-bit storage): the 16 rows of the query tile are 16 HEADS of one token -- they
+// all read the same cached rows, so one key fragment and one staged value tile serve sixteen heads.  Workgroup = (token,
+// block of 16 heads); its four waves take the 32-key steps w, w + 4, ... of the window (which step lands in which wave depends
+// on the token's position alone) with the same step body as the prompt kernel, then merge their running maxima, sums and
+// partial outputs through LDS in wave order, where the sink joins the denominator.
+template <typename P, int NSM, int NVM>
+__global__ __launch_bounds__(256) void lat_decode_mfma_kernel(u16* __restrict__ out, const float* __restrict__ qa, UmbPagedKV kv,
+                                                              const u16* __restrict__ sink, const int* __restrict__ pos,
+                                                              const int* __restrict__ slot_, int H, int Dc, int R, int window,
+                                                              float scale) {
+  extern __shared__ __attribute__((aligned(16))) u16 lat_lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g4 = lane >> 4;
+  const int Dk = Dc + R, LD = Dc + 8;
+  const int ns = (Dk + 31) >> 5, nv = Dc >> 4;
+  u16* v_s = lat_lds + (long)wave * (32 * LD + 32 * 4);
+  long* offs = reinterpret_cast<long*>(v_s + 32 * LD);
+  const int t = blockIdx.x, h = blockIdx.y * 16 + j;
+  const bool h_ok = h < H;
+  const int i = pos[t], slot = slot_[t];
+  const int j_lo = i - window + 1 > 0 ? i - window + 1 : 0;
+  const int total = i - j_lo + 1;
+  const u16* kbase = reinterpret_cast<const u16*>(kv.k);
+  u32x4 qf[NSM];
+  f32x4 o[NVM];
+  {
+    const float* qr = qa + ((long)t * H + (h_ok ? h : H - 1)) * Dk;
+#pragma unroll
+    for (int s = 0; s < NSM; ++s) {
+      const int d = 32 * s + 8 * g4;
+      qf[s] = u32x4{0u, 0u, 0u, 0u};
+      if (s < ns && d < Dk) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(qr + d), c = *reinterpret_cast<const f32x4*>(qr + d + 4);
+        qf[s] = u32x4{pack2<P>(a[0], a[1]), pack2<P>(a[2], a[3]), pack2<P>(c[0], c[1]), pack2<P>(c[2], c[3])};
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < NVM; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  float m_run = -INFINITY, l_run = 0.f;
+  const int nch = Dc >> 3;
+  for (int base = wave * 32; base < total; base += 128) {
+    if (lane < 32) {
+      const int kx = base + lane;
+      offs[lane] = kx < total ? pkv_tok(kv, slot, j_lo + kx, 0, 1, Dk) : -1;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    {
+      // lane = (key row m, parity of the 16-byte chunk); eight chunks of the row in flight before any is written
+      const int m = lane & 31, c0 = lane >> 5;
+      const long offm = offs[m];
+      for (int cb = 0; cb < nch; cb += 16) {
+        u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int ch = cb + c0 + 2 * u;
+          v[u] = (ch < nch && offm >= 0) ? *reinterpret_cast<const u32x4*>(kbase + offm + 8 * ch) : u32x4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int ch = cb + c0 + 2 * u;
+          if (ch < nch) *reinterpret_cast<u32x4*>(v_s + m * LD + 8 * ch) = v[u];
+        }
+      }
+    }
+    f32x4 sc[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      sc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const long off = offs[16 * u + j];
+      const u16* kr = kbase + (off >= 0 ? off : 0);
+      u32x4 kf[NSM];
+#pragma unroll
+      for (int s = 0; s < NSM; ++s) {
+        const int d = 32 * s + 8 * g4;
+        kf[s] = (s < ns && d < Dk && off >= 0) ? *reinterpret_cast<const u32x4*>(kr + d) : u32x4{0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+      for (int s = 0; s < NSM; ++s) {
+        if (s < ns) sc[u] = P::mfma(kf[s], qf[s], sc[u]);
+      }
+    }
+    float sv[8], mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const bool vis = base + 16 * u + 4 * g4 + rr < total;
+        sv[4 * u + rr] = vis ? sc[u][rr] * scale : -INFINITY;
+        mx = fmaxf(mx, sv[4 * u + rr]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);                       // finite: every step a wave runs has a key
+    const float fac = expf(m_run - m_new);
+    float w[8], sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      w[e] = sv[e] == -INFINITY ? 0.f : expf(sv[e] - m_new);
+      sum += w[e];
+    }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    l_run = l_run * fac + sum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < NVM; ++dt) {
+      if (dt < nv) { o[dt][0] *= fac; o[dt][1] *= fac; o[dt][2] *= fac; o[dt][3] *= fac; }
+    }
+    const u32x4 pf = u32x4{pack2<P>(w[0], w[1]), pack2<P>(w[2], w[3]), pack2<P>(w[4], w[5]), pack2<P>(w[6], w[7])};
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int dt = 0; dt < NVM; ++dt) {
+      if (dt < nv) {
+        unsigned e[8];
+#pragma unroll
+        for (int m = 0; m < 8; ++m) e[m] = v_s[((m >> 2) * 16 + 4 * g4 + (m & 3)) * LD + 16 * dt + j];
+        const u32x4 va = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+        o[dt] = P::mfma(va, pf, o[dt]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  // merge the four waves: the value tiles are done with, their LDS holds [4][nv][64] partial tiles and [4][16] (max, sum)
+  __syncthreads();
+  f32x4* part = reinterpret_cast<f32x4*>(lat_lds);
+  float* ml = reinterpret_cast<float*>(part + 4 * nv * 64);
+#pragma unroll
+  for (int dt = 0; dt < NVM; ++dt) {
+    if (dt < nv) part[(wave * nv + dt) * 64 + lane] = o[dt];
+  }
+  if (g4 == 0) { ml[(wave * 16 + j) * 2] = m_run; ml[(wave * 16 + j) * 2 + 1] = l_run; }
+  __syncthreads();
+  if (!h_ok) return;
+  const float sk = sink ? P::to_f(sink[h]) : -INFINITY;
+  float M = sk, f[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) M = fmaxf(M, ml[(w * 16 + j) * 2]);
+  float L = sink ? expf(sk - M) : 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float mw = ml[(w * 16 + j) * 2];
+    f[w] = mw == -INFINITY ? 0.f : expf(mw - M);
+    L += ml[(w * 16 + j) * 2 + 1] * f[w];
+  }
+  const float inv = 1.f / L;
+  for (int dt = wave; dt < nv; dt += 4) {
+    f32x4 a = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const f32x4 pv = part[(w * nv + dt) * 64 + lane];
+      a[0] += pv[0] * f[w]; a[1] += pv[1] * f[w]; a[2] += pv[2] * f[w]; a[3] += pv[3] * f[w];
+    }
+    u32x2 pk;
+    pk[0] = pack2<P>(a[0] * inv, a[1] * inv);
+    pk[1] = pack2<P>(a[2] * inv, a[3] * inv);
+    *reinterpret_cast<u32x2*>(out + ((long)t * H + h) * Dc + 16 * dt + 4 * g4) = pk;
+  }
+}
+
 extern "C" int umb_lat_attend_tiled_ok(int H, int kv_rank, int rot_dim, int dtype) {
   const int Dk = kv_rank + rot_dim;
   return H >= 1 && (dtype == UMB_SEQ_BF16 || dtype == UMB_SEQ_F16) && kv_rank >= 16 && kv_rank % 16 == 0 && kv_rank <= 512 &&
@@ -505,3 +612,99 @@ extern "C" int umb_lat_attend_tiled(void* out, const float* qa, const UmbPagedKV
   UMB_LAUNCH_CHECK();
   return UMB_OK;
 }
+
+extern "C" int umb_lat_prep(void* cq, const UmbPagedKV* kv, const float* proj, int ld, const void* w_q, const void* w_kv,
+                            const int* pos, const int* slot, const float* freq, int T, int q_rank, int kv_rank, int rot_dim,
+                            int rot_dims, float eps, int dtype, hipStream_t st) {
+  if (T < 1 || q_rank < 1 || kv_rank < 1 || rot_dim < 0 || rot_dims < 0 || rot_dims > rot_dim || (rot_dims & 1) || !cq ||
+      !lat_kv_ok(kv) || !proj || !w_q || !w_kv || !pos || !slot || (rot_dims && !freq) || ld < q_rank + kv_rank + rot_dim)
+    return UMB_EINVAL;
+  DISPATCH_SEQ_DTYPE(dtype, {
+    typedef typename El<P>::type E;
+    hipLaunchKernelGGL(lat_prep_kernel<P>, dim3((unsigned)(2L * T)), dim3(256), 0, st, (E*)cq, *kv, proj, ld,
+                       (const E*)w_q, (const E*)w_kv, pos, slot, freq, T, q_rank, kv_rank, rot_dim, rot_dims, eps);
+  })
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_lat_qsplit(void* qn, float* qa, const float* q, const int* pos, const float* freq, int T, int H, int D, int R,
+                              int kv_rank, int rot_dims, int dtype, hipStream_t st) {
+  if (T < 1 || H < 1 || D < 1 || R < 0 || kv_rank < 1 || rot_dims < 0 || rot_dims > R || (rot_dims & 1) || !qn || !qa || !q ||
+      !pos || (rot_dims && !freq))
+    return UMB_EINVAL;
+  const long n = (long)T * H * (D + (R + 1) / 2);
+  DISPATCH_SEQ_DTYPE(dtype, {
+    typedef typename El<P>::type E;
+    hipLaunchKernelGGL(lat_qsplit_kernel<P>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (E*)qn, qa, q, pos, freq, T, H,
+                       D, R, kv_rank, rot_dims);
+  })
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
+extern "C" int umb_lat_attend(void* out, const float* qa, const UmbPagedKV* kv, const void* sink, const int* pos, const int* slot,
+                              int T, int H, int kv_rank, int rot_dim, int window, float scale, int dtype, hipStream_t st) {
+  if (T < 1 || H < 1 || kv_rank < 1 || kv_rank > 64 * LAT_MAXC || rot_dim < 0 || window < 1 || !out || !qa || !lat_kv_ok(kv) ||
+      !pos || !slot)
+    return UMB_EINVAL;
+  // Few tokens: the vector-pipe kernel below spreads a token's keys over sixteen waves and its heads over several workgroups
+  // and finishes sooner; from a few dozen tokens on the chip is full either way and sharing each key fragment among sixteen
+  // heads wins (batch 128 at 1024 keys, kv_rank 512: 1.17 ms a step against 2.40).  UMB_LAT_DEC_MIN moves the switch.
+  const char* env = getenv("UMB_LAT_DEC_MIN");
+  const int lat_dec_min = env ? atoi(env) : 48;
+  if (H >= 4 && T >= lat_dec_min && umb_lat_attend_tiled_ok(H, kv_rank, rot_dim, dtype)) {
+    // 16-bit storage: sixteen heads of a token form the query tile of the matrix-pipe kernel
+    const int Dk = kv_rank + rot_dim;
+    const size_t tiles = 4 * (size_t)(32 * (kv_rank + 8) + 128) * sizeof(u16);
+    const size_t parts = (size_t)4 * (kv_rank / 16) * 64 * sizeof(f32x4) + 4 * 16 * 2 * sizeof(float);
+    const size_t lds = tiles > parts ? tiles : parts;
+    const dim3 grid(T, (H + 15) / 16);
+#define LAT_DEC(NSM, NVM)                                                                                                  \
+  do {                                                                                                                     \
+    if (ensure_dynamic_lds<lat_decode_mfma_kernel<P, NSM, NVM>>(lds) != UMB_OK) return UMB_EHIP;                           \
+    hipLaunchKernelGGL((lat_decode_mfma_kernel<P, NSM, NVM>), grid, dim3(256), lds, st, (u16*)out, qa, *kv,                \
+                       (const u16*)sink, pos, slot, H, kv_rank, rot_dim, window, scale);                                   \
+  } while (0)
+#define LAT_DEC_SHAPE()                                                                                                    \
+  if (Dk <= 128 && kv_rank <= 128) LAT_DEC(4, 8); else if (Dk <= 320 && kv_rank <= 256) LAT_DEC(10, 16); else LAT_DEC(18, 32)
+    if (dtype == UMB_SEQ_BF16) { using P = BF16; LAT_DEC_SHAPE(); }
+    else { using P = F16; LAT_DEC_SHAPE(); }
+#undef LAT_DEC_SHAPE
+#undef LAT_DEC
+    UMB_LAUNCH_CHECK();
+    return UMB_OK;
+  }
+  const int Dk = kv_rank + rot_dim, Dp = (Dk + 3) & ~3;
+  // heads of one workgroup: all of them share the keys, so as many as the register budget of the partial sums allows
+  const int nc = (kv_rank + 63) / 64;
+  int rh = nc <= 2 ? 8 : (nc <= 4 ? 4 : 2);
+  while (rh > 1 && rh / 2 >= H) rh >>= 1;
+  const int hb = (H + rh - 1) / rh;
+  const dim3 grid(T, hb);
+  int nw = (long)T * hb < 1024 ? 16 : 4;
+  auto lds_of = [&](int w) { return ((size_t)w * rh * Dp + (size_t)w * 2 * rh + (size_t)w * (rh * 64 + 128)) * sizeof(float); };
+  if (nw == 16 && lds_of(16) > 128 * 1024) nw = 4;
+  if (lds_of(nw) > 160 * 1024) return UMB_EINVAL;
+  const size_t lds = lds_of(nw);
+#define LAT_LAUNCH(RH, NC, NW)                                                                                            \
+  do {                                                                                                                    \
+    if (ensure_dynamic_lds<lat_attend_kernel<P, RH, NC, NW>>(lds) != UMB_OK) return UMB_EHIP;                             \
+    hipLaunchKernelGGL((lat_attend_kernel<P, RH, NC, NW>), grid, dim3(NW * 64), lds, st, (E*)out, qa, *kv, (const E*)sink, \
+                       pos, slot, T, H, kv_rank, rot_dim, window, scale);                                                 \
+  } while (0)
+#define LAT_NW(RH, NC)                                                                                                    \
+  if (nw == 16) LAT_LAUNCH(RH, NC, 16); else LAT_LAUNCH(RH, NC, 4)
+  DISPATCH_SEQ_DTYPE(dtype, {
+    typedef typename El<P>::type E;
+    if (nc <= 1) { if (rh == 8) { LAT_NW(8, 1); } else if (rh == 4) { LAT_NW(4, 1); } else if (rh == 2) { LAT_NW(2, 1); } else { LAT_NW(1, 1); } }
+    else if (nc <= 2) { if (rh == 8) { LAT_NW(8, 2); } else if (rh == 4) { LAT_NW(4, 2); } else if (rh == 2) { LAT_NW(2, 2); } else { LAT_NW(1, 2); } }
+    else if (nc <= 4) { if (rh == 4) { LAT_NW(4, 4); } else if (rh == 2) { LAT_NW(2, 4); } else { LAT_NW(1, 4); } }
+    else { if (rh == 2) { LAT_NW(2, 8); } else { LAT_NW(1, 8); } }
+  })
+#undef LAT_NW
+#undef LAT_LAUNCH
+  UMB_LAUNCH_CHECK();
+  return UMB_OK;
+}
+
