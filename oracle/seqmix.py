@@ -201,7 +201,8 @@ def routed_experts(X, w_router, experts, top: int, shared=None, margins=None):
     s = torch.sigmoid(z)
     out = torch.zeros_like(X)
     for t in range(X.shape[0]):
-        ranked = sorted(range(len(experts)), key=lambda e: (-float(s[t, e]), e))
+        # ranked on the logits: the same order as on the scores, also where the sigmoid has saturated to 1.0
+        ranked = sorted(range(len(experts)), key=lambda e: (-float(z[t, e]), e))
         order = ranked[:top]
         if margins is not None and top < len(experts):
             margins.append(float((z[t, ranked[top - 1]] - z[t, ranked[top]]) / z[t].std().clamp_min(1e-30)))

@@ -346,7 +346,7 @@ def _lat_oracle(X, w, dtype, **kw):
 
 LAT_CASES = [  # H, D, R, E, q_rank, kv_rank, window, rot_dims, page
     (3, 8, 4, 6, 10, 12, 5, 4, 4), (5, 6, 6, 10, 7, 9, 1, 4, 3), (1, 3, 2, 5, 3, 70, 4, 2, 5), (9, 16, 8, 24, 48, 136, 70, 8, 16),
-    (2, 32, 16, 8, 24, 264, 0, 16, 64), (4, 16, 0, 16, 8, 32, 7, 0, 4), (16, 8, 8, 8, 16, 64, 33, 8, 8)]
+    (2, 32, 16, 8, 24, 264, 0, 16, 64), (4, 16, 0, 16, 8, 32, 7, 0, 4), (16, 8, 8, 8, 16, 64, 33, 8, 8), (3, 8, 8, 8, 16, 600, 20, 8, 8)]
 
 
 @pytest.mark.parametrize("H,D,R,E,q_rank,kv_rank,window,rot_dims,page", LAT_CASES)

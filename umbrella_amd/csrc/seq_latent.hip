@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256) void lat_qsplit_kernel(typename El<P>::type* _
 // denominator per head (the usual rescaling when the maximum grows); the waves' partial results are merged through LDS in
 // wave order together with the sink.  Which keys land in which wave and round depends on the query's position alone -- never
 // on the batch or on how the prompt was cut.
-constexpr int LAT_MAXC = 8;      // value columns per lane: kv_rank <= 512
+constexpr int LAT_MAXC = 16;     // value columns per lane: kv_rank <= 1024
 
 template <typename P, int RH, int NC, int NW>
 __global__ __launch_bounds__(NW * 64) void lat_attend_kernel(typename El<P>::type* __restrict__ out, const float* __restrict__ qa,
@@ -678,7 +678,7 @@ extern "C" int umb_lat_attend(void* out, const float* qa, const UmbPagedKV* kv, 
   const int Dk = kv_rank + rot_dim, Dp = (Dk + 3) & ~3;
   // heads of one workgroup: all of them share the keys, so as many as the register budget of the partial sums allows
   const int nc = (kv_rank + 63) / 64;
-  int rh = nc <= 2 ? 8 : (nc <= 4 ? 4 : 2);
+  int rh = nc <= 2 ? 8 : (nc <= 4 ? 4 : (nc <= 8 ? 2 : 1));
   while (rh > 1 && rh / 2 >= H) rh >>= 1;
   const int hb = (H + rh - 1) / rh;
   const dim3 grid(T, hb);
@@ -700,7 +700,8 @@ extern "C" int umb_lat_attend(void* out, const float* qa, const UmbPagedKV* kv, 
     if (nc <= 1) { if (rh == 8) { LAT_NW(8, 1); } else if (rh == 4) { LAT_NW(4, 1); } else if (rh == 2) { LAT_NW(2, 1); } else { LAT_NW(1, 1); } }
     else if (nc <= 2) { if (rh == 8) { LAT_NW(8, 2); } else if (rh == 4) { LAT_NW(4, 2); } else if (rh == 2) { LAT_NW(2, 2); } else { LAT_NW(1, 2); } }
     else if (nc <= 4) { if (rh == 4) { LAT_NW(4, 4); } else if (rh == 2) { LAT_NW(2, 4); } else { LAT_NW(1, 4); } }
-    else { if (rh == 2) { LAT_NW(2, 8); } else { LAT_NW(1, 8); } }
+    else if (nc <= 8) { if (rh == 2) { LAT_NW(2, 8); } else { LAT_NW(1, 8); } }
+    else { LAT_NW(1, 16); }
   })
 #undef LAT_NW
 #undef LAT_LAUNCH
