@@ -1,8 +1,11 @@
 """Runtime of the sequence-mixer model family on the HIP path (libumbrella_seq.so, include/umbrella_seq.h).
 
-A model is a LIST of layers, each a token mixer -- windowed attention with pooled blocks, or gated linear attention --
-plus an optional gated feed-forward, wrapped in grouped RMS norms.  The list, every size and every constant come from a
-``SeqMixCfg`` (models/config.py); a design contributes a subclass that names its checkpoint tensors (models/gitopel.py).
+A model is a LIST of layers, each a token mixer -- windowed attention with pooled blocks, gated linear attention, or latent
+attention -- plus an optional feed-forward (gated SiLU, PolyNorm, or routed experts with a shared one).  A sublayer reads either
+a grouped RMS norm of the residual stream or the stream itself through a short causal convolution; its output is normed before
+it is added back.  A layer may use another layer's tensors with a cache and state of its own.  The list, every size and every
+constant come from a ``SeqMixCfg`` (models/config.py); a design contributes a subclass that names its checkpoint tensors
+(models/gitopel.py, models/fidizen.py).
 
 Unlike the tree-decoding ``Llama`` runtime this one serves MANY sequences: a step is a ragged batch (the rows of each
 sequence contiguous, nothing padded), key/value pages and recurrent-state slots are handed out by
