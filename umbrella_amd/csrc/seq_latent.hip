@@ -16,6 +16,8 @@
 #include "seq_common.h"
 #include <cstdlib>
 
+constexpr float LOG2E = 1.4426950408889634f;
+
 static inline bool lat_kv_ok(const UmbPagedKV* kv) { return kv && kv->k && kv->pages && kv->page >= 1 && kv->max_pages >= 1; }
 
 // ---- norms of the two latents, rotation of the shared key part, cache append.  One workgroup per (token, part): part 0 =
@@ -239,12 +241,14 @@ __global__ __launch_bounds__(NW * 64) void lat_attend_kernel(typename El<P>::typ
 }
 
 // ---- prompt attention on the matrix pipe (16-bit storage; Dk a multiple of 8, kv_rank a multiple of 16).
-// Workgroup = (16 consecutive positions of one sequence, a block of 4 HPW heads); wave w owns HPW heads and walks the tile's
-// keys -- from the first position's window start to the last position -- in steps of 32, alone (no workgroup barrier).
-// Per step:  the 32 cached rows' first kv_rank features are copied to the wave's LDS tile (they are the VALUES, needed
-//            transposed below); the step is shared by the wave's HPW heads, which also share every key fragment load;
-//   S^T = K Q^T as two 16-key MFMA tiles per head (A = 16 keys x 32 features straight from the cached rows, B = the queries,
-//         rounded to the storage dtype once, when the tile starts);
+// Workgroup = (16 consecutive positions of one sequence, a block of 4 HPW heads); wave w owns HPW heads.  The tile's keys -- from
+// the first position's window start to the last position -- are walked in steps of 32 by the whole workgroup: the step's 32
+// cached rows (all Dk features) are staged ONCE into a shared LDS tile and serve every head of the workgroup, as keys and as
+// values; the next step's rows are already in flight (in registers) while the current one is used, so the one global round
+// trip of a step hides behind its matrix products, and the small tile leaves room for several workgroups per CU.
+// Per step and head:
+//   S^T = K Q^T as two 16-key MFMA tiles (A = 16 keys x 32 features read from the LDS tile, B = the queries, rounded to the
+//         storage dtype once, when the tile starts);
 //   online softmax in fp32: lane (query j, key quad g) holds keys 4g .. 4g+3 of both tiles; the row maximum and sum are
 //         finished over the four lanes of a query by two shuffles; accumulators are rescaled when the maximum grows;
 //   O^T += V^T P^T: the lane's eight weights ARE its share of the B operand when V^T's k index runs over (tile 0: 4g .. 4g+3,
@@ -258,16 +262,18 @@ __global__ __launch_bounds__(256) void lat_attend_mfma_kernel(u16* __restrict__ 
                                                               const int* __restrict__ seq_len, int H, int Dc, int R, int window,
                                                               float scale) {
   extern __shared__ __attribute__((aligned(16))) u16 lat_lds[];
+  constexpr int NLD = (NSM + 1) / 2;                  // 16-byte chunks of a row per staging thread: Dk / 8 chunks over 8 threads
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g4 = lane >> 4;
-  const int Dk = Dc + R, LD = Dc + 8;                 // LDS row stride: 16 bytes of padding spread the key quads over the banks
-  const int ns = (Dk + 31) >> 5, nv = Dc >> 4;
-  u16* v_s = lat_lds + (long)wave * (32 * LD + 32 * 4);       // [32][LD] values, [32] 64-bit offsets
-  long* offs = reinterpret_cast<long*>(v_s + 32 * LD);
+  const int Dk = Dc + R, LD = Dk + 8;                 // LDS row stride: 16 bytes of padding spread the key quads over the banks
+  const int ns = (Dk + 31) >> 5, nv = Dc >> 4, nch = Dk >> 3;
+  constexpr int LT = 36;                              // row stride of the transposed tile: 32 keys + 8 bytes of padding
+  u16* v_s = lat_lds;                                 // [32][LD]: the step's rows as cached (keys: A operand of S^T = K Q^T)
+  u16* v_t = lat_lds + 32 * LD;                       // [Dc][LT]: their first Dc features transposed (values: A operand of O^T)
   const int b = blockIdx.y;
   const int n = seq_len[b], q0 = blockIdx.x * 16;
-  if (q0 >= n) return;
+  if (q0 >= n) return;                                // the whole workgroup
   const int h0 = (blockIdx.z * 4 + wave) * HPW;
-  if (h0 >= H) return;
+  const bool active = h0 < H;                         // a wave without heads still stages rows and meets the barriers
   const int slot = seq_slot[b], row0 = seq_row0[b], pos0 = seq_pos0[b];
   const int nq = n - q0 < 16 ? n - q0 : 16;
   const int i_first = pos0 + q0, i_last = i_first + nq - 1;
@@ -276,6 +282,7 @@ __global__ __launch_bounds__(256) void lat_attend_mfma_kernel(u16* __restrict__ 
   const long qrow = row0 + q0 + (q_ok ? j : nq - 1);
   const int j_lo = i_first - window + 1 > 0 ? i_first - window + 1 : 0;
   const int total = i_last - j_lo + 1;
+  const float scale2 = scale * LOG2E;
   const u16* kbase = reinterpret_cast<const u16*>(kv.k);
   u32x4 qf[HPW][NSM];
   f32x4 o[HPW][NVM];
@@ -284,7 +291,7 @@ __global__ __launch_bounds__(256) void lat_attend_mfma_kernel(u16* __restrict__ 
 #pragma unroll
   for (int hh = 0; hh < HPW; ++hh) {
     h_ok[hh] = h0 + hh < H;
-    const float* qr = qa + (qrow * H + (h_ok[hh] ? h0 + hh : h0)) * Dk;
+    const float* qr = qa + (qrow * H + (h_ok[hh] ? h0 + hh : H - 1)) * Dk;
 #pragma unroll
     for (int s = 0; s < NSM; ++s) {
       const int d = 32 * s + 8 * g4;
@@ -299,112 +306,115 @@ __global__ __launch_bounds__(256) void lat_attend_mfma_kernel(u16* __restrict__ 
     m_run[hh] = -INFINITY;
     l_run[hh] = 0.f;
   }
-  const int nch = Dc >> 3;                            // 16-byte chunks of a value row
-  for (int base = 0; base < total; base += 32) {
-    if (lane < 32) {
-      const int kx = base + lane;
-      offs[lane] = kx < total ? pkv_tok(kv, slot, j_lo + kx, 0, 1, Dk) : -1;
+  // staging role of a thread: key row sm of the step, 16-byte chunks sc, sc + 8, ... of that row
+  const int sm = threadIdx.x & 31, sc = threadIdx.x >> 5;
+  u32x4 stage[NLD];
+  auto fetch = [&](int base) {
+    const int kx = base + sm;
+    const long off = kx < total ? pkv_tok(kv, slot, j_lo + kx, 0, 1, Dk) : -1;
+#pragma unroll
+    for (int u = 0; u < NLD; ++u) {
+      const int ch = sc + 8 * u;
+      stage[u] = (off >= 0 && ch < nch) ? *reinterpret_cast<const u32x4*>(kbase + off + 8 * ch) : u32x4{0u, 0u, 0u, 0u};
     }
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    {
-      // lane = (key row m, parity of the 16-byte chunk); eight chunks of the row in flight before any is written
-      const int m = lane & 31, c0 = lane >> 5;
-      const long offm = offs[m];
-      for (int cb = 0; cb < nch; cb += 16) {
-        u32x4 v[8];
+  };
+  fetch(0);
+  for (int base = 0; base < total; base += 32) {
+    __syncthreads();                                  // every wave is done with the previous tile
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int ch = cb + c0 + 2 * u;
-          v[u] = (ch < nch && offm >= 0) ? *reinterpret_cast<const u32x4*>(kbase + offm + 8 * ch) : u32x4{0u, 0u, 0u, 0u};
-        }
+    for (int u = 0; u < NLD; ++u) {
+      const int ch = sc + 8 * u;
+      if (ch < nch) {
+        *reinterpret_cast<u32x4*>(v_s + sm * LD + 8 * ch) = stage[u];
+        if (8 * ch < Dc) {                            // Dc is a multiple of 16: a chunk is all values or all rotated key part
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int ch = cb + c0 + 2 * u;
-          if (ch < nch) *reinterpret_cast<u32x4*>(v_s + m * LD + 8 * ch) = v[u];
+          for (int e = 0; e < 4; ++e) {
+            v_t[(8 * ch + 2 * e) * LT + sm] = (u16)(stage[u][e] & 0xffffu);
+            v_t[(8 * ch + 2 * e + 1) * LT + sm] = (u16)(stage[u][e] >> 16);
+          }
         }
       }
     }
-    f32x4 sc[HPW][2];
+    __syncthreads();
+    if (base + 32 < total) fetch(base + 32);          // in flight while this step is used
+    if (!active) continue;
+    f32x4 sc2[HPW][2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
 #pragma unroll
-      for (int hh = 0; hh < HPW; ++hh) sc[hh][u] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const long off = offs[16 * u + j];
-      const u16* kr = kbase + (off >= 0 ? off : 0);
-      u32x4 kf[NSM];
+      for (int hh = 0; hh < HPW; ++hh) sc2[hh][u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const u16* kr = v_s + (16 * u + j) * LD;
 #pragma unroll
       for (int s = 0; s < NSM; ++s) {
         const int d = 32 * s + 8 * g4;
-        kf[s] = (s < ns && d < Dk && off >= 0) ? *reinterpret_cast<const u32x4*>(kr + d) : u32x4{0u, 0u, 0u, 0u};
-      }
-#pragma unroll
-      for (int s = 0; s < NSM; ++s) {
         if (s < ns) {
+          const u32x4 kf = d < Dk ? *reinterpret_cast<const u32x4*>(kr + d) : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-          for (int hh = 0; hh < HPW; ++hh) sc[hh][u] = P::mfma(kf[s], qf[hh][s], sc[hh][u]);
+          for (int hh = 0; hh < HPW; ++hh) sc2[hh][u] = P::mfma(kf, qf[hh][s], sc2[hh][u]);
         }
       }
+    }
+    // which of the lane's eight keys this query sees: the same for every head
+    bool vis[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int jt = j_lo + base + 16 * (e >> 2) + 4 * g4 + (e & 3);
+      vis[e] = q_ok && jt <= i_j && jt > i_j - window;
     }
     u32x4 pf[HPW];
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
+      // maxima and exponents in base 2 (scale2 = scale log2 e): one v_exp_f32 per weight
       float sv[8], mx = -INFINITY;
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int jt = j_lo + base + 16 * u + 4 * g4 + rr;
-          const bool vis = q_ok && jt <= i_j && jt > i_j - window;
-          sv[4 * u + rr] = vis ? sc[hh][u][rr] * scale : -INFINITY;
-          mx = fmaxf(mx, sv[4 * u + rr]);
-        }
+      for (int e = 0; e < 8; ++e) {
+        sv[e] = vis[e] ? sc2[hh][e >> 2][e & 3] * scale2 : -INFINITY;
+        mx = fmaxf(mx, sv[e]);
+      }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run[hh], mx);
-      const float fac = m_new == -INFINITY ? 1.f : expf(m_run[hh] - m_new);
+      const float m_ref = m_new == -INFINITY ? 0.f : m_new;          // a row that has seen no key yet: all weights 0
+      const float fac = __builtin_amdgcn_exp2f(m_run[hh] - m_ref);
       float w[8], sum = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        w[e] = sv[e] == -INFINITY ? 0.f : expf(sv[e] - m_new);
+        w[e] = __builtin_amdgcn_exp2f(sv[e] - m_ref);
         sum += w[e];
       }
       sum += __shfl_xor(sum, 16, 64);
       sum += __shfl_xor(sum, 32, 64);
       l_run[hh] = l_run[hh] * fac + sum;
       m_run[hh] = m_new;
+      if (__ballot(fac != 1.f)) {                                    // the maximum moved for some row of the tile
 #pragma unroll
-      for (int dt = 0; dt < NVM; ++dt) {
-        if (dt < nv) { o[hh][dt][0] *= fac; o[hh][dt][1] *= fac; o[hh][dt][2] *= fac; o[hh][dt][3] *= fac; }
+        for (int dt = 0; dt < NVM; ++dt) {
+          if (dt < nv) { o[hh][dt][0] *= fac; o[hh][dt][1] *= fac; o[hh][dt][2] *= fac; o[hh][dt][3] *= fac; }
+        }
       }
       pf[hh] = u32x4{pack2<P>(w[0], w[1]), pack2<P>(w[2], w[3]), pack2<P>(w[4], w[5]), pack2<P>(w[6], w[7])};
     }
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    // O^T[d][query] += V^T[d][keys] P^T[keys][query]: lane (d row j of tile dt, quad g4) gathers its 8 keys' values
+    // O^T[d][query] += V^T[d][keys] P^T[keys][query]: lane (d row j of tile dt, quad g4) reads its 8 keys' values
 #pragma unroll
     for (int dt = 0; dt < NVM; ++dt) {
       if (dt < nv) {
-        unsigned e[8];
-#pragma unroll
-        for (int m = 0; m < 8; ++m) e[m] = v_s[((m >> 2) * 16 + 4 * g4 + (m & 3)) * LD + 16 * dt + j];
-        const u32x4 va = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+        const u16* vr = v_t + (16 * dt + j) * LT + 4 * g4;
+        const u32x2 t0 = *reinterpret_cast<const u32x2*>(vr), t1 = *reinterpret_cast<const u32x2*>(vr + 16);
+        const u32x4 va = u32x4{t0[0], t0[1], t1[0], t1[1]};
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) o[hh][dt] = P::mfma(va, pf[hh], o[hh][dt]);
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-    __builtin_amdgcn_wave_barrier();
   }
   // lane holds O^T[d = 16 dt + 4 g4 + rr][query j]
-  if (q_ok) {
+  if (q_ok && active) {
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
       if (!h_ok[hh]) continue;
-      const float sk = sink ? P::to_f(sink[h0 + hh]) : -INFINITY;
+      const float sk = sink ? P::to_f(sink[h0 + hh]) * LOG2E : -INFINITY;      // the running maximum is in base 2
       const float M = fmaxf(m_run[hh], sk);
-      const float f = expf(m_run[hh] - M);
-      const float inv = f / (l_run[hh] * f + (sink ? expf(sk - M) : 0.f));
+      const float f = exp2f(m_run[hh] - M);
+      const float inv = f / (l_run[hh] * f + (sink ? exp2f(sk - M) : 0.f));
 #pragma unroll
       for (int dt = 0; dt < NVM; ++dt) {
         if (dt < nv) {
@@ -439,6 +449,7 @@ __global__ __launch_bounds__(256) void lat_decode_mfma_kernel(u16* __restrict__ 
   const int i = pos[t], slot = slot_[t];
   const int j_lo = i - window + 1 > 0 ? i - window + 1 : 0;
   const int total = i - j_lo + 1;
+  const float scale2 = scale * LOG2E;
   const u16* kbase = reinterpret_cast<const u16*>(kv.k);
   u32x4 qf[NSM];
   f32x4 o[NVM];
@@ -500,32 +511,34 @@ __global__ __launch_bounds__(256) void lat_decode_mfma_kernel(u16* __restrict__ 
         if (s < ns) sc[u] = P::mfma(kf[s], qf[s], sc[u]);
       }
     }
-    float sv[8], mx = -INFINITY;
+    float sv[8], mx = -INFINITY;                                // maxima and exponents in base 2: one v_exp_f32 per weight
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const bool vis = base + 16 * u + 4 * g4 + rr < total;
-        sv[4 * u + rr] = vis ? sc[u][rr] * scale : -INFINITY;
+        sv[4 * u + rr] = vis ? sc[u][rr] * scale2 : -INFINITY;
         mx = fmaxf(mx, sv[4 * u + rr]);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);                       // finite: every step a wave runs has a key
-    const float fac = expf(m_run - m_new);
+    const float fac = __builtin_amdgcn_exp2f(m_run - m_new);
     float w[8], sum = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      w[e] = sv[e] == -INFINITY ? 0.f : expf(sv[e] - m_new);
+      w[e] = __builtin_amdgcn_exp2f(sv[e] - m_new);
       sum += w[e];
     }
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
     l_run = l_run * fac + sum;
     m_run = m_new;
+    if (__ballot(fac != 1.f)) {
 #pragma unroll
-    for (int dt = 0; dt < NVM; ++dt) {
-      if (dt < nv) { o[dt][0] *= fac; o[dt][1] *= fac; o[dt][2] *= fac; o[dt][3] *= fac; }
+      for (int dt = 0; dt < NVM; ++dt) {
+        if (dt < nv) { o[dt][0] *= fac; o[dt][1] *= fac; o[dt][2] *= fac; o[dt][3] *= fac; }
+      }
     }
     const u32x4 pf = u32x4{pack2<P>(w[0], w[1]), pack2<P>(w[2], w[3]), pack2<P>(w[4], w[5]), pack2<P>(w[6], w[7])};
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
@@ -554,15 +567,15 @@ __global__ __launch_bounds__(256) void lat_decode_mfma_kernel(u16* __restrict__ 
   if (g4 == 0) { ml[(wave * 16 + j) * 2] = m_run; ml[(wave * 16 + j) * 2 + 1] = l_run; }
   __syncthreads();
   if (!h_ok) return;
-  const float sk = sink ? P::to_f(sink[h]) : -INFINITY;
+  const float sk = sink ? P::to_f(sink[h]) * LOG2E : -INFINITY;          // the running maxima are in base 2
   float M = sk, f[4];
 #pragma unroll
   for (int w = 0; w < 4; ++w) M = fmaxf(M, ml[(w * 16 + j) * 2]);
-  float L = sink ? expf(sk - M) : 0.f;
+  float L = sink ? exp2f(sk - M) : 0.f;
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
     const float mw = ml[(w * 16 + j) * 2];
-    f[w] = mw == -INFINITY ? 0.f : expf(mw - M);
+    f[w] = mw == -INFINITY ? 0.f : exp2f(mw - M);
     L += ml[(w * 16 + j) * 2 + 1] * f[w];
   }
   const float inv = 1.f / L;
@@ -593,7 +606,7 @@ extern "C" int umb_lat_attend_tiled(void* out, const float* qa, const UmbPagedKV
       !umb_lat_attend_tiled_ok(H, kv_rank, rot_dim, dtype))
     return UMB_EINVAL;
   const int Dk = kv_rank + rot_dim;
-  const size_t lds = 4 * (size_t)(32 * (kv_rank + 8) + 128) * sizeof(u16);
+  const size_t lds = ((size_t)32 * (Dk + 8) + (size_t)kv_rank * 36) * sizeof(u16);
 #define LAT_MFMA(NSM, NVM, HPW)                                                                                            \
   do {                                                                                                                     \
     const dim3 grid((max_len + 15) / 16, B, (H + 4 * HPW - 1) / (4 * HPW));                                                \
@@ -603,7 +616,7 @@ extern "C" int umb_lat_attend_tiled(void* out, const float* qa, const UmbPagedKV
   } while (0)
 #define LAT_MFMA_SHAPE()                                                                                                   \
   if (Dk <= 128 && kv_rank <= 128) { if (H >= 8) LAT_MFMA(4, 8, 2); else LAT_MFMA(4, 8, 1); }                              \
-  else if (Dk <= 320 && kv_rank <= 256) { if (H >= 8) LAT_MFMA(10, 16, 2); else LAT_MFMA(10, 16, 1); }                     \
+  else if (Dk <= 320 && kv_rank <= 256) LAT_MFMA(10, 16, 1);   /* two heads a wave spill to AGPRs here: measured slower */ \
   else LAT_MFMA(18, 32, 1)
   if (dtype == UMB_SEQ_BF16) { using P = BF16; LAT_MFMA_SHAPE(); }
   else { using P = F16; LAT_MFMA_SHAPE(); }
